@@ -1,0 +1,170 @@
+"""ctypes binding of the gfx950 shared library (include/archscale_muon.h).
+
+There is no fallback: if the library is missing or a call fails, this raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Dict, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .build import LIB_PATH
+
+# enums of include/archscale_muon.h
+DTYPE_BF16, DTYPE_F32 = 0, 1
+EPS_ADD, EPS_CLAMP = 0, 1
+PREC_BF16, PREC_BF16_BSPLIT = 0, 1
+NS_CAST_INPUT_FIRST = 1
+CHUNK_ELEMS = 8192
+ABI_VERSION = 1
+
+#: numpy layouts of muon_pre_item / muon_post_item (natural C alignment)
+PRE_ITEM = np.dtype(
+    [("g", "<u8"), ("m", "<u8"), ("u", "<u8"), ("w", "<u8"), ("numel", "<i8"),
+     ("g_dtype", "<i4"), ("m_dtype", "<i4"), ("u_dtype", "<i4"), ("w_dtype", "<i4")], align=True)
+POST_ITEM = np.dtype(
+    [("w", "<u8"), ("u", "<u8"), ("numel", "<i8"), ("lr_ratio", "<f4"), ("w_dtype", "<i4")], align=True)
+assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32
+
+
+class MuonLibraryError(RuntimeError):
+    """The HIP library is missing, has the wrong ABI, or a call into it failed."""
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+
+_SIGNATURES = {
+    "muon_abi_version": (ctypes.c_int, []),
+    "muon_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "muon_ns_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
+    "muon_ns_batched": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_ns_flops": (None, [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 3),
+    "muon_syrk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
+    "muon_syrk": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float,
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_momentum": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+        ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_void_p]),
+    "muon_update_plain": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+        ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_void_p]),
+    "muon_muonh_scratch_floats": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int]),
+    "muon_update_muonh": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+        ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once; raise if it is not built or has another ABI."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise MuonLibraryError(
+                f"{LIB_PATH} is not built; run `python -m archscale_amd.build` (needs hipcc). "
+                "There is no PyTorch or CPU fallback for the Muon kernels.")
+        try:
+            handle = ctypes.CDLL(LIB_PATH)
+        except OSError as e:  # pragma: no cover - depends on the machine
+            raise MuonLibraryError(f"cannot load {LIB_PATH}: {e}") from e
+        for name, (res, args) in _SIGNATURES.items():
+            try:
+                fn = getattr(handle, name)
+            except AttributeError as e:
+                raise MuonLibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
+            fn.restype = res
+            fn.argtypes = args
+        got = handle.muon_abi_version()
+        if got != ABI_VERSION:
+            raise MuonLibraryError(f"{LIB_PATH} has ABI {got}, this package needs {ABI_VERSION}; rebuild it")
+        _lib = handle
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = lib().muon_status_string(status).decode()
+        if status < 0:
+            raise ValueError(f"{what}: {msg}")
+        raise MuonLibraryError(f"{what}: HIP error {status}: {msg}")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return DTYPE_BF16
+    if dt == torch.float32:
+        return DTYPE_F32
+    raise TypeError(f"the Muon kernels take bfloat16 or float32 tensors, got {dt}")
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_cuda(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise MuonLibraryError(
+            f"{what} is on {t.device}: the Muon kernels run on an AMD GPU only (no CPU fallback)")
+
+
+# ---------------------------------------------------------------------------
+# workspace: one growing byte buffer per (device, tag); torch owns the memory
+# ---------------------------------------------------------------------------
+_workspaces: Dict[Tuple[int, str], torch.Tensor] = {}
+
+
+def workspace(device: torch.device, nbytes: int, tag: str = "ns") -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            del _workspaces[key]
+            del buf
+        buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def release_workspaces() -> None:
+    """Drop the cached workspaces (they are re-created on demand)."""
+    _workspaces.clear()
+
+
+_abc_cache: Dict[Tuple, ctypes.Array] = {}
+
+
+def abc_array(coeffs: Sequence[Tuple[float, float, float]]):
+    key = tuple((float(a), float(b), float(c)) for a, b, c in coeffs)
+    arr = _abc_cache.get(key)
+    if arr is None:
+        flat = [v for row in key for v in row]
+        arr = (ctypes.c_float * len(flat))(*flat)
+        _abc_cache[key] = arr
+    return arr
+
+
+def ns_flops(batch: int, rows: int, cols: int, iters: int, prec_mode: int) -> Tuple[float, float, float]:
+    """(dense, symmetric, issued) FLOP counts of one muon_ns_batched call."""
+    d, s, i = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    lib().muon_ns_flops(batch, rows, cols, iters, prec_mode, ctypes.byref(d), ctypes.byref(s), ctypes.byref(i))
+    return d.value, s.value, i.value

@@ -1,0 +1,43 @@
+// Internal interface between the HBM-bound kernels and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/archscale_muon.h"
+
+namespace archscale {
+
+enum { DT_BF16 = MUON_DTYPE_BF16, DT_F32 = MUON_DTYPE_F32 };
+enum { EPS_ADD = MUON_EPS_ADD, EPS_CLAMP = MUON_EPS_CLAMP };
+
+typedef muon_pre_item PreItem;
+typedef muon_post_item PostItem;
+
+struct MomentumCoef {
+  float mm, mg, um, ug, l2;
+};
+
+hipError_t launch_momentum(const PreItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                           MomentumCoef c, hipStream_t stream);
+
+// per-matrix Frobenius norms of in[batch][rows][cols] -> scale[b] = 1/(|X|+eps) or 1/max(|X|,eps)
+hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch,
+                             int rows, int cols, float eps, int eps_mode, float* partial, float* scale,
+                             hipStream_t stream);
+
+// D = bf16(scale*in) in the input's orientation and T = its transpose (T may be null), both zero-padded to
+// d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).
+hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
+                         int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
+                         void* T, long t_bstride, int ldt, hipStream_t stream);
+
+hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
+                             int batch, int rows, int cols, hipStream_t stream);
+
+hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                             float lr, float lrwd, int cautious, hipStream_t stream);
+
+hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream);
+
+}  // namespace archscale

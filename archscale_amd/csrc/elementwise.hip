@@ -1,0 +1,500 @@
+// HBM-bound kernels of the Muon / MuonH step for gfx950: multi-tensor momentum,
+// Frobenius norms, normalise + transpose into the padded Newton-Schulz workspace,
+// and the plain-Muon / MuonH weight updates.
+//
+// All multi-tensor kernels are driven by a device table of items (one contiguous
+// range each) and a prefix array of chunk counts: block c finds its item by binary
+// search, so ONE launch covers every matrix of every shape (replaces the
+// per-parameter compiled foreach graphs of lit_gpt/optim/muon.py:653-818).
+// Reductions are two-stage and ordered (per-chunk partials, then one block per
+// item sums them in index order), so results do not depend on scheduling.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "elementwise.h"
+
+namespace archscale {
+
+static constexpr int EW_THREADS = 256;
+static constexpr int EW_VEC = 8;                                   // elements per thread per trip
+static constexpr int EW_TRIPS = MUON_CHUNK_ELEMS / (EW_THREADS * EW_VEC);
+static_assert(EW_TRIPS * EW_THREADS * EW_VEC == MUON_CHUNK_ELEMS, "chunk must be a whole number of trips");
+
+// ---------------------------------------------------------------------------
+// small helpers
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint16_t f2bf(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ float bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+template <int DT> struct Elem;  // DT_BF16 / DT_F32 access of 8 consecutive elements
+template <> struct Elem<DT_BF16> {
+  typedef uint16_t T;
+  static __device__ __forceinline__ void load8(const void* p, long i, float (&v)[8]) {
+    const uint4 r = *(const uint4*)((const uint16_t*)p + i);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { v[2 * k] = bf2f(w[k] & 0xffff); v[2 * k + 1] = bf2f(w[k] >> 16); }
+  }
+  static __device__ __forceinline__ void store8(void* p, long i, const float (&v)[8]) {
+    uint4 r;
+    r.x = f2bf(v[0]) | ((uint32_t)f2bf(v[1]) << 16);
+    r.y = f2bf(v[2]) | ((uint32_t)f2bf(v[3]) << 16);
+    r.z = f2bf(v[4]) | ((uint32_t)f2bf(v[5]) << 16);
+    r.w = f2bf(v[6]) | ((uint32_t)f2bf(v[7]) << 16);
+    *(uint4*)((uint16_t*)p + i) = r;
+  }
+  static __device__ __forceinline__ float load1(const void* p, long i) { return bf2f(((const uint16_t*)p)[i]); }
+  static __device__ __forceinline__ void store1(void* p, long i, float v) { ((uint16_t*)p)[i] = f2bf(v); }
+  static __device__ __forceinline__ float round(float v) { return bf2f(f2bf(v)); }
+};
+template <> struct Elem<DT_F32> {
+  typedef float T;
+  static __device__ __forceinline__ void load8(const void* p, long i, float (&v)[8]) {
+    const float4 a = *(const float4*)((const float*)p + i);
+    const float4 b = *(const float4*)((const float*)p + i + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store8(void* p, long i, const float (&v)[8]) {
+    *(float4*)((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4*)((float*)p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+  static __device__ __forceinline__ float load1(const void* p, long i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ void store1(void* p, long i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+__device__ __forceinline__ bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+// item that owns global chunk c: largest i with prefix[i] <= c
+__device__ __forceinline__ int find_item(const int32_t* __restrict__ prefix, int n_items, int c) {
+  int lo = 0, hi = n_items;  // invariant: prefix[lo] <= c < prefix[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (prefix[mid] <= c) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ordered block reduction of up to 3 values; result valid in thread 0
+template <int N>
+__device__ __forceinline__ void block_reduce(float (&v)[N], float* smem /* N * 4 floats */) {
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_down(v[k], off, 64);
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) smem[k * 4 + w] = v[k];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) v[k] = (smem[k * 4 + 0] + smem[k * 4 + 1]) + (smem[k * 4 + 2] + smem[k * 4 + 3]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 1. momentum:  M <- c_mm*M + c_mg*G ;  U <- c_um*M + c_ug*G   (G optionally += l2*W first)
+//    lit_gpt: (mu, 1, mu|1, 1|0)  (muon.py:665-679);  emerging: (b, 1-b, b|1, 1-b|0)
+//    (orthogonalized_optimizer.py:193-199, mixin.py:48-49 for the l2 term)
+// ---------------------------------------------------------------------------
+template <int GD, int MD, int UD>
+__device__ __forceinline__ void momentum_range(const PreItem& it, long begin, long end, const MomentumCoef c, bool vec_ok) {
+  const void* g = it.g; void* m = it.m; void* u = it.u;
+  if (vec_ok) {
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float gv[8], mv[8], uv[8];
+        Elem<GD>::load8(g, i, gv);
+        Elem<MD>::load8(m, i, mv);
+        if (c.l2 != 0.f) {
+          float wv[8];
+          if (it.w_dtype == DT_BF16) Elem<DT_BF16>::load8(it.w, i, wv); else Elem<DT_F32>::load8(it.w, i, wv);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) gv[k] = Elem<GD>::round(gv[k] + c.l2 * wv[k]);
+          Elem<GD>::store8(const_cast<void*>(g), i, gv);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float gm = Elem<MD>::round(gv[k]);            // G cast to M's dtype (muon.py:666)
+          const float mn = Elem<MD>::round(c.mm * mv[k] + c.mg * gm);
+          mv[k] = mn;
+          uv[k] = c.um * mn + c.ug * gm;
+        }
+        Elem<MD>::store8(m, i, mv);
+        Elem<UD>::store8(u, i, uv);
+      }
+    }
+  } else {
+    for (long i = begin + threadIdx.x; i < end; i += EW_THREADS) {
+      float gv = Elem<GD>::load1(g, i);
+      if (c.l2 != 0.f) {
+        const float wv = it.w_dtype == DT_BF16 ? Elem<DT_BF16>::load1(it.w, i) : Elem<DT_F32>::load1(it.w, i);
+        gv = Elem<GD>::round(gv + c.l2 * wv);
+        Elem<GD>::store1(const_cast<void*>(g), i, gv);
+      }
+      const float gm = Elem<MD>::round(gv);
+      const float mn = Elem<MD>::round(c.mm * Elem<MD>::load1(m, i) + c.mg * gm);
+      Elem<MD>::store1(m, i, mn);
+      Elem<UD>::store1(u, i, c.um * mn + c.ug * gm);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+momentum_kernel(const PreItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items, MomentumCoef c) {
+  const int chunk = blockIdx.x;
+  const int ii = find_item(prefix, n_items, chunk);
+  const PreItem it = items[ii];
+  const long begin = (long)(chunk - prefix[ii]) * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
+  const bool vec_ok = aligned16(it.g) && aligned16(it.m) && aligned16(it.u) && (c.l2 == 0.f || aligned16(it.w)) &&
+                      (it.numel % EW_VEC == 0);
+  const int key = (it.g_dtype << 2) | (it.m_dtype << 1) | it.u_dtype;
+  switch (key) {
+    case 0: momentum_range<DT_BF16, DT_BF16, DT_BF16>(it, begin, end, c, vec_ok); break;
+    case 1: momentum_range<DT_BF16, DT_BF16, DT_F32>(it, begin, end, c, vec_ok); break;
+    case 2: momentum_range<DT_BF16, DT_F32, DT_BF16>(it, begin, end, c, vec_ok); break;
+    case 3: momentum_range<DT_BF16, DT_F32, DT_F32>(it, begin, end, c, vec_ok); break;
+    case 4: momentum_range<DT_F32, DT_BF16, DT_BF16>(it, begin, end, c, vec_ok); break;
+    case 5: momentum_range<DT_F32, DT_BF16, DT_F32>(it, begin, end, c, vec_ok); break;
+    case 6: momentum_range<DT_F32, DT_F32, DT_BF16>(it, begin, end, c, vec_ok); break;
+    default: momentum_range<DT_F32, DT_F32, DT_F32>(it, begin, end, c, vec_ok); break;
+  }
+}
+
+hipError_t launch_momentum(const PreItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                           MomentumCoef c, hipStream_t stream) {
+  if (total_chunks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(momentum_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items, c);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// 2. per-matrix Frobenius norm of a strided batch -> scale[b] = 1/(|X|+eps) or 1/max(|X|,eps)
+//    (muon.py:883-888; F.normalize semantics for spectral_ball_utils.py:46)
+// ---------------------------------------------------------------------------
+template <int DT, bool CAST_FIRST>
+__global__ void __launch_bounds__(EW_THREADS)
+sumsq_partial_kernel(const void* __restrict__ in, long batch_stride, int rows, int cols, int ld,
+                     int chunks_per_mat, float* __restrict__ partial) {
+  __shared__ float red[4];
+  const int b = blockIdx.y, chunk = blockIdx.x;
+  const char* base = (const char*)in + (size_t)b * batch_stride * sizeof(typename Elem<DT>::T);
+  const long numel = (long)rows * cols;
+  const long begin = (long)chunk * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < numel ? begin + MUON_CHUNK_ELEMS : numel;
+  float s[1] = {0.f};
+  const bool dense = (ld == cols);
+  if (dense && aligned16(base) && numel % EW_VEC == 0) {
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float v[8];
+        Elem<DT>::load8(base, i, v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float x = CAST_FIRST ? bf2f(f2bf(v[k])) : v[k]; s[0] += x * x; }
+      }
+    }
+  } else {
+    for (long i = begin + threadIdx.x; i < end; i += EW_THREADS) {
+      const long r = i / cols, cc = i - r * cols;
+      float x = Elem<DT>::load1(base, r * ld + cc);
+      if (CAST_FIRST) x = bf2f(f2bf(x));
+      s[0] += x * x;
+    }
+  }
+  block_reduce<1>(s, red);
+  if (threadIdx.x == 0) partial[(size_t)b * chunks_per_mat + chunk] = s[0];
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+norm_scale_kernel(const float* __restrict__ partial, int chunks_per_mat, float eps, int eps_mode,
+                  float* __restrict__ scale) {
+  __shared__ float red[4];
+  const int b = blockIdx.x;
+  float s[1] = {0.f};
+  for (int i = threadIdx.x; i < chunks_per_mat; i += EW_THREADS) s[0] += partial[(size_t)b * chunks_per_mat + i];
+  block_reduce<1>(s, red);
+  if (threadIdx.x == 0) {
+    const float n = sqrtf(s[0]);
+    scale[b] = eps_mode == EPS_ADD ? 1.f / (n + eps) : 1.f / fmaxf(n, eps);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 3. normalise + lay out:  D[b][r][c] = bf16(s_b * in[b][r][c]),  T[b][c][r] = same value,
+//    both zero-padded to the tile multiples the GEMMs assume (replaces the
+//    X/(norm+eps), .mT and .contiguous() of newton_schulz_triton.py:358-366).
+// ---------------------------------------------------------------------------
+template <int DT, bool CAST_FIRST>
+__global__ void __launch_bounds__(256)
+normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, int cols, int ld,
+                        const float* __restrict__ scale,
+                        uint16_t* __restrict__ D, long d_bstride, int ldd, int d_rows, int d_cols,
+                        uint16_t* __restrict__ T, long t_bstride, int ldt) {
+  // 64x64 tile; d_rows/d_cols are the padded extents (multiples of 64)
+  __shared__ uint16_t tile[64][66];
+  const int b = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const char* base = (const char*)in + (size_t)b * in_bstride * sizeof(typename Elem<DT>::T);
+  const float s = scale ? scale[b] : 1.f;
+  const int tr = threadIdx.x >> 3;        // 0..31
+  const int tc = (threadIdx.x & 7) * 8;   // 0..56
+  const bool vec = aligned16(base) && (ld % 8 == 0) && (in_bstride % 8 == 0);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = r0 + tr + h * 32, c = c0 + tc;
+    float v[8];
+    if (r < rows && c + 7 < cols && vec) {
+      Elem<DT>::load8(base, (long)r * ld + c, v);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = (r < rows && c + k < cols) ? Elem<DT>::load1(base, (long)r * ld + c + k) : 0.f;
+    }
+    uint16_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float x = CAST_FIRST ? bf2f(f2bf(v[k])) : v[k];
+      o[k] = f2bf(x * s);
+      tile[tr + h * 32][tc + k] = o[k];
+    }
+    if (r < d_rows && c < d_cols) {
+      uint4 pk;
+      pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
+      pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
+      *(uint4*)(D + (size_t)b * d_bstride + (size_t)r * ldd + c) = pk;
+    }
+  }
+  if (!T) return;
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = c0 + tr + h * 32;  // row of T
+    const int r = r0 + tc;           // 8 consecutive columns of T
+    uint16_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = tile[tc + k][tr + h * 32];
+    if (c < d_cols && r < d_rows) {
+      uint4 pk;
+      pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
+      pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
+      *(uint4*)(T + (size_t)b * t_bstride + (size_t)c * ldt + r) = pk;
+    }
+  }
+}
+
+hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch,
+                             int rows, int cols, float eps, int eps_mode, float* partial, float* scale,
+                             hipStream_t stream) {
+  const long numel = (long)rows * cols;
+  const int cpm = (int)((numel + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
+  if (batch > 65535) return hipErrorInvalidValue;
+  dim3 g1(cpm, batch);
+#define ARCHSCALE_SS(DT, CF)                                                                                  \
+  hipLaunchKernelGGL((sumsq_partial_kernel<DT, CF>), g1, dim3(EW_THREADS), 0, stream, in, in_bstride, rows,   \
+                     cols, ld, cpm, partial)
+  if (in_dtype == DT_BF16) ARCHSCALE_SS(DT_BF16, false);
+  else if (cast_first) ARCHSCALE_SS(DT_F32, true);
+  else ARCHSCALE_SS(DT_F32, false);
+#undef ARCHSCALE_SS
+  hipLaunchKernelGGL(norm_scale_kernel, dim3(batch), dim3(EW_THREADS), 0, stream, partial, cpm, eps, eps_mode,
+                     scale);
+  return hipGetLastError();
+}
+
+hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
+                         int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
+                         void* T, long t_bstride, int ldt, hipStream_t stream) {
+  if (batch > 65535 || d_rows / 64 > 65535 || d_rows % 64 || d_cols % 64) return hipErrorInvalidValue;
+  dim3 g3(d_cols / 64, d_rows / 64, batch);
+#define ARCHSCALE_NL(DT, CF)                                                                                   \
+  hipLaunchKernelGGL((normalize_layout_kernel<DT, CF>), g3, dim3(256), 0, stream, in, in_bstride, rows, cols,  \
+                     ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride, ldt)
+  if (in_dtype == DT_BF16) ARCHSCALE_NL(DT_BF16, false);
+  else if (cast_first) ARCHSCALE_NL(DT_F32, true);
+  else ARCHSCALE_NL(DT_F32, false);
+#undef ARCHSCALE_NL
+  return hipGetLastError();
+}
+
+// strided copy of the leading rows x cols corner of a padded bf16 buffer into a caller tensor
+__global__ void __launch_bounds__(256)
+unpad_copy_kernel(const uint16_t* __restrict__ src, long s_bstride, int lds_, uint16_t* __restrict__ dst,
+                  long d_bstride, int ldd, int rows, int cols) {
+  const int b = blockIdx.z;
+  const int r = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  if (r < rows && c < cols) dst[(size_t)b * d_bstride + (size_t)r * ldd + c] = src[(size_t)b * s_bstride + (size_t)r * lds_ + c];
+}
+
+hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
+                             int batch, int rows, int cols, hipStream_t stream) {
+  if (batch > 65535 || (rows + 3) / 4 > 65535) return hipErrorInvalidValue;
+  dim3 g((cols + 63) / 64, (rows + 3) / 4, batch);
+  hipLaunchKernelGGL(unpad_copy_kernel, g, dim3(256), 0, stream, (const uint16_t*)src, s_bstride, lds_,
+                     (uint16_t*)dst, d_bstride, ldd, rows, cols);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// 4. weight updates
+//    x' = weight-decayed x (muon.py:703-718): plain x*(1-lr*wd), or cautious
+//         x - lr*wd*x*[x*u >= 0]
+//    plain Muon   X <- x' - lr*ratio*U                              (muon.py:720-722)
+//    MuonH        X <- r*(x' - lr*s*U), s=|x'|/max(|U|,eps), r=|x'|/max(|x'-lr*s*U|,eps)
+//                                                                   (muon.py:614-639, 725-818)
+//    MuonH needs |x'|^2, |U|^2, <x',U> first; |x'-tU|^2 follows in closed form.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float decayed(float x, float u, float lrwd, int cautious) {
+  if (cautious) return (x * u >= 0.f) ? x - lrwd * x : x;
+  return x * (1.f - lrwd);
+}
+
+template <int WD>
+__device__ __forceinline__ void post_reduce_range(const PostItem& it, long begin, long end, float lrwd, int cautious,
+                                                  bool vec_ok, float (&s)[3]) {
+  if (vec_ok) {
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float x[8], u[8];
+        Elem<WD>::load8(it.w, i, x);
+        Elem<DT_BF16>::load8(it.u, i, u);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float xd = decayed(x[k], u[k], lrwd, cautious);
+          s[0] += xd * xd; s[1] += u[k] * u[k]; s[2] += xd * u[k];
+        }
+      }
+    }
+  } else {
+    for (long i = begin + threadIdx.x; i < end; i += EW_THREADS) {
+      const float u = Elem<DT_BF16>::load1(it.u, i);
+      const float xd = decayed(Elem<WD>::load1(it.w, i), u, lrwd, cautious);
+      s[0] += xd * xd; s[1] += u * u; s[2] += xd * u;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+post_reduce_kernel(const PostItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
+                   float lrwd, int cautious, float* __restrict__ partial /* [total_chunks][3] */) {
+  __shared__ float red[12];
+  const int chunk = blockIdx.x;
+  const int ii = find_item(prefix, n_items, chunk);
+  const PostItem it = items[ii];
+  const long begin = (long)(chunk - prefix[ii]) * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
+  const bool vec_ok = aligned16(it.w) && aligned16(it.u) && (it.numel % EW_VEC == 0);
+  float s[3] = {0.f, 0.f, 0.f};
+  if (it.w_dtype == DT_BF16) post_reduce_range<DT_BF16>(it, begin, end, lrwd, cautious, vec_ok, s);
+  else post_reduce_range<DT_F32>(it, begin, end, lrwd, cautious, vec_ok, s);
+  block_reduce<3>(s, red);
+  if (threadIdx.x == 0) {
+    partial[(size_t)chunk * 3 + 0] = s[0];
+    partial[(size_t)chunk * 3 + 1] = s[1];
+    partial[(size_t)chunk * 3 + 2] = s[2];
+  }
+}
+
+// one block per item: (alpha, beta) with X <- alpha*x' + beta*U
+__global__ void __launch_bounds__(EW_THREADS)
+muonh_coef_kernel(const int32_t* __restrict__ prefix, const float* __restrict__ partial, float lr, float eps,
+                  float2* __restrict__ coef) {
+  __shared__ double red[3][4];
+  const int ii = blockIdx.x;
+  double s[3] = {0.0, 0.0, 0.0};
+  for (int c = prefix[ii] + threadIdx.x; c < prefix[ii + 1]; c += EW_THREADS) {
+    s[0] += partial[(size_t)c * 3 + 0];
+    s[1] += partial[(size_t)c * 3 + 1];
+    s[2] += partial[(size_t)c * 3 + 2];
+  }
+#pragma unroll
+  for (int k = 0; k < 3; ++k)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s[k] += __shfl_down(s[k], off, 64);
+  if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = s[0]; red[1][threadIdx.x >> 6] = s[1]; red[2][threadIdx.x >> 6] = s[2]; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const double xx = red[0][0] + red[0][1] + red[0][2] + red[0][3];
+    const double uu = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+    const double xu = red[2][0] + red[2][1] + red[2][2] + red[2][3];
+    const double xn = sqrt(xx), un = sqrt(uu);
+    const double e = (double)eps;
+    const double t = (double)lr * xn / (un > e ? un : e);            // step along U
+    double yy = xx - 2.0 * t * xu + t * t * uu;                      // |x' - tU|^2
+    if (yy < 0.0) yy = 0.0;
+    const double yn = sqrt(yy);
+    const double r = xn / (yn > e ? yn : e);
+    coef[ii] = make_float2((float)r, (float)(-r * t));
+  }
+}
+
+template <int WD, bool HAS_COEF>
+__device__ __forceinline__ void post_apply_range(const PostItem& it, long begin, long end, float lrwd, int cautious,
+                                                 bool vec_ok, float alpha, float beta) {
+  if (vec_ok) {
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float x[8], u[8];
+        Elem<WD>::load8(it.w, i, x);
+        Elem<DT_BF16>::load8(it.u, i, u);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[k] = alpha * decayed(x[k], u[k], lrwd, cautious) + beta * u[k];
+        Elem<WD>::store8(it.w, i, x);
+      }
+    }
+  } else {
+    for (long i = begin + threadIdx.x; i < end; i += EW_THREADS) {
+      const float u = Elem<DT_BF16>::load1(it.u, i);
+      Elem<WD>::store1(it.w, i, alpha * decayed(Elem<WD>::load1(it.w, i), u, lrwd, cautious) + beta * u);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+post_apply_kernel(const PostItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
+                  float lr, float lrwd, int cautious, const float2* __restrict__ coef) {
+  const int chunk = blockIdx.x;
+  const int ii = find_item(prefix, n_items, chunk);
+  const PostItem it = items[ii];
+  const long begin = (long)(chunk - prefix[ii]) * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
+  const bool vec_ok = aligned16(it.w) && aligned16(it.u) && (it.numel % EW_VEC == 0);
+  float alpha = 1.f, beta = -lr * it.lr_ratio;
+  if (coef) { const float2 c = coef[ii]; alpha = c.x; beta = c.y; }
+  if (it.w_dtype == DT_BF16) post_apply_range<DT_BF16, true>(it, begin, end, lrwd, cautious, vec_ok, alpha, beta);
+  else post_apply_range<DT_F32, true>(it, begin, end, lrwd, cautious, vec_ok, alpha, beta);
+}
+
+hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                             float lr, float lrwd, int cautious, hipStream_t stream) {
+  if (total_chunks <= 0) return hipSuccess;
+  hipLaunchKernelGGL(post_apply_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
+                     lr, lrwd, cautious, (const float2*)nullptr);
+  return hipGetLastError();
+}
+
+hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream) {
+  if (total_chunks <= 0) return hipSuccess;
+  float* partial = scratch;                                             // 3 * total_chunks
+  float2* coef = (float2*)(scratch + (size_t)3 * total_chunks + ((total_chunks & 1) ? 1 : 0));  // 8-byte aligned
+  hipLaunchKernelGGL(post_reduce_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
+                     lrwd, cautious, partial);
+  hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), dim3(EW_THREADS), 0, stream, prefix, partial, lr, eps, coef);
+  hipLaunchKernelGGL(post_apply_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
+                     lr, lrwd, cautious, (const float2*)coef);
+  return hipGetLastError();
+}
+
+}  // namespace archscale

@@ -1,0 +1,37 @@
+// Internal interface between the Newton-Schulz GEMM kernels and the C-ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace archscale {
+
+enum { MODE_SYRK = 0, MODE_SYRK2 = 1, MODE_BX = 2 };
+
+// C[m][n] = sum_k P[m][k] * Q[n][k]; all leading dimensions / strides in elements.
+struct GemmParams {
+  const __bf16* P;   // [batch][tilesM*BM][ldp]
+  const __bf16* P2;  // second pass over K for P (low half of a split B), or null
+  const __bf16* Q;   // [batch][tilesN*BN][ldq]
+  long strideP, strideQ;
+  int ldp, ldq;
+  int K;             // reduction length, multiple of 64
+  int tilesM, tilesN;
+  int batch;
+  const __bf16* E;   // epilogue addend, read as E[col][row..row+3]
+  long strideE;
+  int lde;
+  __bf16* C;         // row-major output [row][col] (may be null in MODE_BX)
+  __bf16* C2;        // low half of a split output (MODE_SYRK2 with split)
+  long strideC;
+  int ldc;
+  __bf16* Ct;        // transposed output [col][row] (MODE_BX, may be null)
+  long strideCt;
+  int ldct;
+  float alpha, beta;
+  int m_valid, n_valid;  // true extents for the bounds-checked final store
+};
+
+// tile: 256 (256x256 block tile, 8 waves) or 128 (128x128, 4 waves)
+hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream);
+
+}  // namespace archscale

@@ -1,0 +1,140 @@
+/* C ABI of the MI355X (gfx950) Muon / MuonH hot path.
+ *
+ * Plain pointers and sizes only: every pointer named *_dev is DEVICE memory owned by
+ * the caller; the library never allocates or frees device memory and never
+ * synchronises the host.  All work is enqueued on the stream argument (a
+ * hipStream_t passed as void*; NULL = the default stream).
+ *
+ * Return value of every int function: 0 = success, < 0 = MUON_E_* argument error,
+ * > 0 = a hipError_t from a launch.  Nothing throws or aborts.
+ *
+ * Reference file:line citations are relative to the microsoft/ArchScale checkout.
+ */
+#ifndef ARCHSCALE_MUON_H
+#define ARCHSCALE_MUON_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MUON_ABI_VERSION 1
+
+/* element types of caller tensors */
+#define MUON_DTYPE_BF16 0
+#define MUON_DTYPE_F32 1
+
+/* how eps enters the Frobenius normalisation */
+#define MUON_EPS_ADD 0   /* X / (|X| + eps)      lit_gpt/optim/muon.py:888 */
+#define MUON_EPS_CLAMP 1 /* X / max(|X|, eps)    emerging_optimizers/.../spectral_ball_utils.py:46 */
+
+/* precision of B = bA + cA^2 as an operand of B*X */
+#define MUON_PREC_BF16 0       /* one bf16 rounding per GEMM epilogue (rounding points of newton_schulz_triton.py:374-378) */
+#define MUON_PREC_BF16_BSPLIT 1 /* B kept as a bf16 hi+lo pair, B*X accumulates both (needed for the constant-coefficient table) */
+
+/* flags of muon_ns_batched */
+#define MUON_NS_CAST_INPUT_FIRST 1 /* fp32 input: round to bf16 BEFORE taking the norm (muon.py:883-888); default is
+                                      normalise in fp32, then round (spectral_ball_utils.py:46-54) */
+
+#define MUON_E_ARG (-1)        /* null pointer, non-positive extent, bad enum */
+#define MUON_E_WORKSPACE (-2)  /* workspace too small or misaligned */
+#define MUON_E_UNSUPPORTED (-3)
+
+/* elements covered by one block of the multi-tensor kernels; chunk prefixes are in these units */
+#define MUON_CHUNK_ELEMS 8192
+
+int muon_abi_version(void);
+const char* muon_status_string(int status);
+
+/* ---- Newton-Schulz -------------------------------------------------------------------------
+ * Replaces zeropower_via_newtonschulz5 (lit_gpt/optim/muon.py:869-897, lit_gpt/legacy_optim.py:187-213),
+ * newton_schulz_triton (lit_gpt/optim/newton_schulz_triton.py:344-382: ns_line_1, ns_line_2, addmm/baddbmm),
+ * _small_msign (emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:37-74) and
+ * newton_schulz / newton_schulz_step_tsyrk (.../muon_utils.py:68-164, 262-287).
+ *
+ * in  : [batch] matrices of rows x cols, leading dimension in_ld, batch stride in_batch_stride (elements),
+ *       dtype in_dtype.  Not modified.
+ * out : bf16, same logical shape, leading dimension out_ld, batch stride out_batch_stride.  May alias `in`
+ *       only if in_dtype is bf16 and the strides are equal.
+ * abc : HOST array of 3*iters floats, one (a, b, c) row per iteration (the reference has three different
+ *       tables; none is compiled in).
+ * Each matrix is normalised by its own Frobenius norm, tall matrices (rows > cols) are iterated transposed
+ * and returned in the caller's orientation.
+ * ws  : device workspace of at least muon_ns_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t muon_ns_workspace_bytes(int batch, int rows, int cols, int prec_mode);
+
+int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld,
+                    void* out_dev, int64_t out_batch_stride, int out_ld,
+                    int batch, int rows, int cols,
+                    const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
+                    void* ws_dev, size_t ws_bytes, void* stream);
+
+/* Algorithmic work of one call, for roofline accounting: dense-count FLOPs (what a GEMM library executes),
+ * symmetric-count FLOPs (upper-triangle SYRK minimum) and FLOPs this library issues (tiles incl. padding,
+ * full diagonal tiles and the second pass of the B split). */
+void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
+                   double* dense, double* symmetric, double* issued);
+
+/* ---- single products on caller tensors ------------------------------------------------------
+ * D = alpha * A A^T + beta * C, A [batch] n x k (bf16, row-major, ld lda), C symmetric n x n or NULL, D n x n,
+ * both triangles written.  Replaces ns_line_1 / ns_line_2 (newton_schulz_triton.py:142-178, 269-310) and
+ * tsyrk_ex (emerging_optimizers/triton_kernels/syrk.py:188-261).
+ */
+size_t muon_syrk_workspace_bytes(int batch, int n, int k);
+int muon_syrk(const void* a_dev, int64_t a_batch_stride, int lda,
+              const void* c_dev, int64_t c_batch_stride, int ldc,
+              void* d_dev, int64_t d_batch_stride, int ldd,
+              int batch, int n, int k, float alpha, float beta,
+              void* ws_dev, size_t ws_bytes, void* stream);
+
+/* ---- multi-tensor momentum ------------------------------------------------------------------
+ * For every item:  M <- c_mm*M + c_mg*G ;  U <- c_um*M + c_ug*G   (G rounded to M's dtype first).
+ *   lit_gpt Muon   (lit_gpt/optim/muon.py:653-681):  c_mm=mu, c_mg=1, (c_um,c_ug) = (mu,1) nesterov | (1,0)
+ *   emerging Muon  (emerging_optimizers/.../orthogonalized_optimizer.py:193-199):
+ *                  c_mm=beta, c_mg=1-beta, (c_um,c_ug) = (beta,1-beta) nesterov | (1,0)
+ * l2 != 0 first does G <- G + l2*W in place (emerging_optimizers/mixin.py:48-49).
+ * items/prefix are DEVICE arrays; prefix[i] = first chunk of item i, prefix[n_items] = total_chunks,
+ * an item of numel elements owns ceil(numel / MUON_CHUNK_ELEMS) chunks.
+ */
+typedef struct muon_pre_item {
+  const void* g; /* gradient (read; written only when l2 != 0) */
+  void* m;       /* momentum buffer, in place */
+  void* u;       /* output */
+  const void* w; /* weights, only read when l2 != 0 */
+  int64_t numel;
+  int32_t g_dtype, m_dtype, u_dtype, w_dtype;
+} muon_pre_item;
+
+int muon_momentum(const muon_pre_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                  float c_mm, float c_mg, float c_um, float c_ug, float l2, void* stream);
+
+/* ---- multi-tensor weight updates ------------------------------------------------------------
+ * x' = x*(1 - lr_wd), or with cautious != 0:  x' = x - lr_wd*x where x*u >= 0  (muon.py:703-718).
+ * muon_update_plain:  W <- x' - lr*lr_ratio*U                                   (muon.py:720-722;
+ *                     emerging_optimizers/.../orthogonalized_optimizer.py:225-228 with lr_ratio = scale factor)
+ * muon_update_muonh:  W <- r*(x' - lr*s*U),  s = |x'|/max(|U|,eps),  r = |x'|/max(|x' - lr*s*U|,eps),
+ *                     norms over the whole item                                 (muon.py:614-639, 725-818).
+ * scratch_dev: muon_muonh_scratch_floats(n_items, total_chunks) floats, 8-byte aligned.
+ */
+typedef struct muon_post_item {
+  void* w;       /* weights, in place */
+  const void* u; /* orthogonalised update, bf16 */
+  int64_t numel;
+  float lr_ratio; /* adjusted_lr / lr for this tensor (plain update only) */
+  int32_t w_dtype;
+} muon_post_item;
+
+int muon_update_plain(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                      float lr, float lr_wd, int cautious, void* stream);
+
+size_t muon_muonh_scratch_floats(int n_items, int total_chunks);
+int muon_update_muonh(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                      float lr, float lr_wd, float eps, int cautious, float* scratch_dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARCHSCALE_MUON_H */
