@@ -49,6 +49,10 @@ _SIGNATURES = {
         ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_ns_flops": (None, [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 3),
+    "muon_profile_begin": (ctypes.c_int, []),
+    "muon_profile_collect": (ctypes.c_int, [
+        ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_double),
+        ctypes.POINTER(ctypes.c_double), ctypes.c_int]),
     "muon_syrk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
     "muon_syrk": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
@@ -168,3 +172,25 @@ def ns_flops(batch: int, rows: int, cols: int, iters: int, prec_mode: int) -> Tu
     d, s, i = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
     lib().muon_ns_flops(batch, rows, cols, iters, prec_mode, ctypes.byref(d), ctypes.byref(s), ctypes.byref(i))
     return d.value, s.value, i.value
+
+
+def profile_begin() -> None:
+    check(lib().muon_profile_begin(), "muon_profile_begin")
+
+
+def profile_collect(capacity: int = 4096):
+    """Per-launch records of the Newton-Schulz GEMMs since profile_begin():
+    list of dicts {ms, tile, mode, split, final, flops_algorithmic, flops_issued}."""
+    ms = (ctypes.c_float * capacity)()
+    key = (ctypes.c_int32 * capacity)()
+    fa = (ctypes.c_double * capacity)()
+    fi = (ctypes.c_double * capacity)()
+    n = lib().muon_profile_collect(ms, key, fa, fi, capacity)
+    if n < 0:
+        raise MuonLibraryError(f"muon_profile_collect failed with {n}")
+    out = []
+    for i in range(min(n, capacity)):
+        k = key[i]
+        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool(k & 2), final=bool(k & 1),
+                        flops_algorithmic=fa[i], flops_issued=fi[i]))
+    return out

@@ -4,6 +4,9 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
+#include <vector>
+
 #include "../../include/archscale_muon.h"
 #include "elementwise.h"
 #include "ns_gemm.h"
@@ -60,6 +63,35 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode) {
 }
 
 inline long sym_tiles(int t) { return (long)t * (t + 1) / 2; }
+
+// Optional per-launch timing of the Newton-Schulz GEMMs (muon_profile_begin / muon_profile_collect):
+// one pair of HIP events around every GEMM launch, on the stream the kernel runs on.
+struct ProfRec {
+  hipEvent_t start, stop;
+  int key;  // tile*100 + mode*10 + split*2 + final
+  double flops_algorithmic, flops_issued;
+};
+std::mutex g_prof_mutex;
+std::vector<ProfRec> g_prof;
+bool g_prof_on = false;
+
+hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GemmParams& g, hipStream_t stream,
+                      double flops_algorithmic, double flops_issued) {
+  if (!g_prof_on) return launch_ns_gemm(tile, mode, split, final_, g, stream);
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  ProfRec r;
+  r.key = tile * 100 + mode * 10 + (split ? 2 : 0) + (final_ ? 1 : 0);
+  r.flops_algorithmic = flops_algorithmic;
+  r.flops_issued = flops_issued;
+  hipError_t e;
+  if ((e = hipEventCreate(&r.start)) != hipSuccess) return e;
+  if ((e = hipEventCreate(&r.stop)) != hipSuccess) return e;
+  if ((e = hipEventRecord(r.start, stream)) != hipSuccess) return e;
+  e = launch_ns_gemm(tile, mode, split, final_, g, stream);
+  hipError_t e2 = hipEventRecord(r.stop, stream);
+  g_prof.push_back(r);
+  return e != hipSuccess ? e : e2;
+}
 
 }  // namespace
 
@@ -147,12 +179,16 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
     g.P = X[cur]; g.Q = X[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
     g.tilesM = g.tilesN = tm;
     g.C = A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
-    if ((e = launch_ns_gemm(pl.tile, MODE_SYRK, false, false, g, stream)) != hipSuccess) return (int)e;
+    const double bm = (double)batch, dm = pl.m, dn = pl.n, tl = pl.tile;
+    const double st = (double)sym_tiles(tm);
+    if ((e = timed_gemm(pl.tile, MODE_SYRK, false, false, g, stream, bm * dm * dm * dn,
+                        bm * 2.0 * tl * tl * st * pl.Np)) != hipSuccess) return (int)e;
     // B = c A A + b A
     g.P = A; g.Q = A; g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
     g.E = A; g.strideE = as; g.lde = pl.Mp;
     g.C = Bh; g.C2 = Bl; g.alpha = c; g.beta = b;
-    if ((e = launch_ns_gemm(pl.tile, MODE_SYRK2, split, false, g, stream)) != hipSuccess) return (int)e;
+    if ((e = timed_gemm(pl.tile, MODE_SYRK2, split, false, g, stream, bm * dm * dm * dm,
+                        bm * 2.0 * tl * tl * st * pl.Mp)) != hipSuccess) return (int)e;
     // X' = a X + B X
     g.P = Bh; g.P2 = Bl; g.Q = Xt[cur]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp; g.K = pl.Mp;
     g.tilesM = tm; g.tilesN = tn;
@@ -166,7 +202,8 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
       if (!tall) { g.C = (__bf16*)out_dev; g.strideC = out_batch_stride; g.ldc = out_ld; g.Ct = nullptr; }
       else { g.C = nullptr; g.Ct = (__bf16*)out_dev; g.strideCt = out_batch_stride; g.ldct = out_ld; }
     }
-    if ((e = launch_ns_gemm(pl.tile, MODE_BX, split, last, g, stream)) != hipSuccess) return (int)e;
+    if ((e = timed_gemm(pl.tile, MODE_BX, split, last, g, stream, bm * 2.0 * dm * dm * dn,
+                        bm * 2.0 * tl * tl * tm * tn * pl.Mp * (split ? 2.0 : 1.0))) != hipSuccess) return (int)e;
     cur ^= 1;
   }
   return 0;
@@ -211,6 +248,38 @@ int muon_syrk(const void* a_dev, int64_t a_batch_stride, int lda, const void* c_
   e = launch_ns_gemm(tile, c_dev ? MODE_SYRK2 : MODE_SYRK, false, false, g, stream);
   if (e != hipSuccess) return (int)e;
   return (int)launch_unpad_copy(Dp, (long)Np * Np, Np, d_dev, d_batch_stride, ldd, batch, n, n, stream);
+}
+
+int muon_profile_begin(void) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  for (auto& r : g_prof) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
+  g_prof.clear();
+  g_prof_on = true;
+  return 0;
+}
+
+int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algorithmic_host,
+                         double* flops_issued_host, int capacity) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_on = false;
+  int n = 0;
+  for (auto& r : g_prof) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(r.stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.start, r.stop);
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+    if (e != hipSuccess) { g_prof.clear(); return -(int)e - 1000; }
+    if (n < capacity) {
+      if (ms_host) ms_host[n] = ms;
+      if (key_host) key_host[n] = r.key;
+      if (flops_algorithmic_host) flops_algorithmic_host[n] = r.flops_algorithmic;
+      if (flops_issued_host) flops_issued_host[n] = r.flops_issued;
+    }
+    ++n;
+  }
+  g_prof.clear();
+  return n;
 }
 
 int muon_momentum(const muon_pre_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,

@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Benchmark of the Muon / MuonH hot path on one MI355X.
+
+A "step" is one full MuonH optimizer step (momentum -> Newton-Schulz-5 -> hypersphere update) over every 2-D
+weight of the depth-16 GQA transformer parameter set: 112 bf16 matrices, 721.4 M elements, seeded synthetic
+weights N(0, 0.02^2) and gradients N(0, 1e-3^2), resident in HBM before the timed region.
+
+Prints ONE JSON line: headline = dense-count Newton-Schulz TFLOP/s over the whole step (what a GEMM library
+would execute: 5*(4 m^2 n + 2 m^3) per matrix), ms per step, the roofline of the dominant kernel measured
+with HIP events per launch, and the CPU baseline (the oracle's eager-bf16 restatement of the reference's CPU
+path) timed on a bounded sample in the same run.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+LAYER_SHAPES = [  # one layer of the depth-16 config: Wq, Wk, Wv, Wo, W1, W3, W2
+    (2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (5632, 2048), (5632, 2048), (2048, 5632)]
+N_LAYERS = 16
+
+
+def dense_flops(shape, iters=5):
+    m, n = min(shape), max(shape)
+    return iters * (4.0 * m * m * n + 2.0 * m ** 3)
+
+
+def sym_flops(shape, iters=5):
+    m, n = min(shape), max(shape)
+    return iters * (3.0 * m * m * n + 1.0 * m ** 3)
+
+
+def make_tensors(device, seed, layers=N_LAYERS):
+    g = torch.Generator(device=device).manual_seed(seed)
+    params, grads = [], []
+    for _ in range(layers):
+        for s in LAYER_SHAPES:
+            w = (torch.randn(*s, generator=g, device=device) * 0.02).to(torch.bfloat16)
+            params.append(torch.nn.Parameter(w))
+            grads.append((torch.randn(*s, generator=g, device=device) * 1e-3).to(torch.bfloat16))
+    return params, grads
+
+
+def cpu_baseline(coeffs_name, seed):
+    """The oracle (a port of the reference's eager CPU path: bf16 storage, every op rounds) on ONE layer's
+    tensor set, all host cores."""
+    from oracle import muon_oracle as O
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(seed)
+    Ws = [(torch.randn(*s, generator=g) * 0.02).to(torch.bfloat16) for s in LAYER_SHAPES]
+    Gs = [(torch.randn(*s, generator=g) * 1e-3).to(torch.bfloat16) for s in LAYER_SHAPES]
+    Ms = [torch.zeros_like(w) for w in Ws]
+    coeffs = O.coefficient_schedule(coeffs_name, 5)
+    # untimed warm-up on the smallest matrix
+    O.lit_gpt_muon_step(Ws[1].clone(), Gs[1], Ms[1].clone(), lr=0.02, mu=0.95, wd=0.0, eps=1e-8, nesterov=True,
+                        adjust="spectral_norm", flatten=False, cautious=False, use_muonh=True, coeffs=coeffs,
+                        ns_storage="bf16_eager")
+    t0 = time.perf_counter()
+    for w, gr, m in zip(Ws, Gs, Ms):
+        O.lit_gpt_muon_step(w, gr, m, lr=0.02, mu=0.95, wd=0.0, eps=1e-8, nesterov=True, adjust="spectral_norm",
+                            flatten=False, cautious=False, use_muonh=True, coeffs=coeffs, ns_storage="bf16_eager")
+    dt = time.perf_counter() - t0
+    flops = sum(dense_flops(s) for s in LAYER_SHAPES)
+    return {
+        "value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"1 of {N_LAYERS} layers (7 matrices, {flops / 1e12:.2f} TFLOP dense), one timed pass of the "
+                  f"eager-bf16 oracle, {dt:.1f} s; full step extrapolates to {dt * N_LAYERS * 1e3:.0f} ms",
+        "ms_per_step_extrapolated": round(dt * N_LAYERS * 1e3, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--coeffs", choices=["quintic", "simple"], default="quintic",
+                    help="quintic = the reference's production 5-row schedule; simple = constant row with the B split")
+    ap.add_argument("--layers", type=int, default=N_LAYERS, help="(debug) fewer layers; the result is then not the metric")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=1236)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every box here has one); --gpus must be 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    from archscale_amd import _lib
+    from archscale_amd.optim.muon import Muon
+    import archscale_amd.optim.newton_schulz_hip as H
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    params, grads = make_tensors(dev, args.seed, args.layers)
+    for p, g in zip(params, grads):
+        p.grad = g
+    simple = args.coeffs == "simple"
+    opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, adjust_lr="spectral_norm",
+               use_muonh=True, ns_coefficients=[H.SIMPLE_ROW] * 5 if simple else None,
+               ns_precision="bsplit" if simple else "bf16")
+
+    for _ in range(args.warmup):  # also warms the momentum so that M != G
+        opt.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        opt.step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # one more, instrumented step: HIP events around every phase and every Newton-Schulz GEMM launch
+    opt.phase_events = []
+    _lib.profile_begin()
+    opt.step()
+    torch.cuda.synchronize()
+    recs = _lib.profile_collect()
+    phases = {}
+    for name, a, b in opt.phase_events:
+        phases[name] = phases.get(name, 0.0) + a.elapsed_time(b)
+    opt.phase_events = None
+
+    shapes = [tuple(p.shape) for p in params]
+    n_elem = sum(p.numel() for p in params)
+    f_dense = sum(dense_flops(s) for s in shapes)
+    f_sym = sum(sym_flops(s) for s in shapes)
+
+    # dominant kernel: the X' = aX + BX product in its main (non-final) instantiation
+    by_kernel = {}
+    for r in recs:
+        k = (r["tile"], r["mode"], r["split"], r["final"])
+        d = by_kernel.setdefault(k, dict(n=0, ms=0.0, fa=0.0, fi=0.0))
+        d["n"] += 1; d["ms"] += r["ms"]; d["fa"] += r["flops_algorithmic"]; d["fi"] += r["flops_issued"]
+    names = {0: "syrk", 1: "syrk2", 2: "bx"}
+    kernels = []
+    for (tile, mode, split, final), d in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ms"]):
+        kernels.append({
+            "kernel": f"ns_gemm<{tile},{names[mode]}{',split' if split else ''}{',final' if final else ''}>",
+            "launches_per_step": d["n"], "avg_ms": round(d["ms"] / d["n"], 4),
+            "algorithmic_tflops": round(d["fa"] / d["ms"] / 1e9, 1), "issued_tflops": round(d["fi"] / d["ms"] / 1e9, 1),
+            "ms_per_step": round(d["ms"], 3)})
+    dom_key = max(by_kernel, key=lambda k: by_kernel[k]["ms"])
+    dom = by_kernel[dom_key]
+    achieved = dom["fa"] / dom["ms"] / 1e9
+    roofline = {
+        "bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+        "kernel": f"ns_gemm_kernel<{dom_key[0]},{names[dom_key[1]]}{',split' if dom_key[2] else ''}"
+                  f"{',final' if dom_key[3] else ''}>",
+        "launches": dom["n"], "avg_launch_ms": round(dom["ms"] / dom["n"], 4),
+        "flops_per_launch": dom["fa"] / dom["n"],
+        "issued_frac": round(dom["fi"] / dom["ms"] / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+    }
+    gemm_ms = sum(d["ms"] for d in by_kernel.values())
+    f_issued = sum(d["fi"] for d in by_kernel.values())
+    hbm = {}
+    bytes_per_elem = {"momentum": 8.0, "update_muonh": 10.0, "update_plain": 6.0}
+    for name, ms in phases.items():
+        if name in bytes_per_elem:
+            gbs = n_elem * bytes_per_elem[name] / ms / 1e6
+            hbm[name] = {"ms": round(ms, 3), "GB/s": round(gbs, 0), "frac": round(gbs / HBM_PEAK_GBS, 3),
+                         "bytes_per_elem": bytes_per_elem[name]}
+    ns_ms = sum(ms for n, ms in phases.items() if n.startswith("newton_schulz"))
+
+    out = {
+        "metric": "Muon NS5 TFLOP/s (% bf16 MFMA peak) + MuonH step ms, d16 param set, 1 GPU",
+        "value": round(f_dense / ms_per_step / 1e9, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 2: full MuonH step, depth-{args.layers} GQA transformer, "
+                               f"{len(params)} bf16 matrices, {n_elem / 1e6:.1f} M elements, "
+                               f"mu 0.95 nesterov, NS5 {args.coeffs} coefficients, lr 0.02, seed {args.seed}",
+                   "coefficients": args.coeffs, "ns_precision": "bsplit" if simple else "bf16"},
+        "value_definition": "dense-count NS FLOPs (5*(4m^2n+2m^3) per matrix) / wall time of the WHOLE step",
+        "ns_gemm_pct_mfma_peak_issued": round(f_issued / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
+        "ns_gemm_pct_mfma_peak_symmetric": round(f_sym / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
+        "ns_gemm_ms": round(gemm_ms, 3), "ns_phase_ms": round(ns_ms, 3),
+        "roofline": roofline,
+        "kernels": kernels,
+        "hbm_kernels": hbm,
+        "phases_ms": {k: round(v, 3) for k, v in phases.items()},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.coeffs, args.seed)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -78,6 +78,19 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
 void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
                    double* dense, double* symmetric, double* issued);
 
+/* Per-launch timing of the Newton-Schulz GEMM kernels, for roofline accounting (no counterpart in the
+ * reference).  Between muon_profile_begin() and muon_profile_collect() every GEMM launch of muon_ns_batched is
+ * bracketed by a pair of HIP events on its stream.  muon_profile_collect waits for them, writes up to `capacity`
+ * records to the HOST arrays (any may be NULL) and returns the number of launches recorded (< 0 on error):
+ *   ms                elapsed milliseconds of the launch
+ *   key               tile*100 + mode*10 + split*2 + final  (mode 0 = X X^T, 1 = cAA+bA, 2 = aX + BX)
+ *   flops_algorithmic minimum FLOPs of the product (symmetric products counted once)
+ *   flops_issued      FLOPs of the tiles actually launched
+ */
+int muon_profile_begin(void);
+int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algorithmic_host,
+                         double* flops_issued_host, int capacity);
+
 /* ---- single products on caller tensors ------------------------------------------------------
  * D = alpha * A A^T + beta * C, A [batch] n x k (bf16, row-major, ld lda), C symmetric n x n or NULL, D n x n,
  * both triangles written.  Replaces ns_line_1 / ns_line_2 (newton_schulz_triton.py:142-178, 269-310) and

@@ -1,0 +1,181 @@
+"""CPU-only checks: the shared library loads and exports every symbol the header declares, the ctypes
+layouts match the header's structs, and the host-side logic (grouping, flatten policy, lr ratios,
+constructor validation) behaves like the reference's."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "archscale_muon.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(muon_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from archscale_amd import _lib
+    from archscale_amd.build import LIB_PATH
+    assert os.path.exists(LIB_PATH), "build the library first: python -m archscale_amd.build"
+    handle = _lib.lib()
+    declared = _declared_functions()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(handle, name), f"{name} is declared in the header but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == declared
+    assert handle.muon_abi_version() == 1
+    assert b"success" in handle.muon_status_string(0)
+    assert b"workspace" in handle.muon_status_string(-2)
+
+
+def test_struct_layouts_and_constants_match_header():
+    from archscale_amd import _lib
+    text = open(HEADER).read()
+    assert int(re.search(r"#define MUON_CHUNK_ELEMS (\d+)", text).group(1)) == _lib.CHUNK_ELEMS
+    assert int(re.search(r"#define MUON_ABI_VERSION (\d+)", text).group(1)) == _lib.ABI_VERSION
+
+    class Pre(ctypes.Structure):
+        _fields_ = [("g", ctypes.c_void_p), ("m", ctypes.c_void_p), ("u", ctypes.c_void_p), ("w", ctypes.c_void_p),
+                    ("numel", ctypes.c_int64), ("g_dtype", ctypes.c_int32), ("m_dtype", ctypes.c_int32),
+                    ("u_dtype", ctypes.c_int32), ("w_dtype", ctypes.c_int32)]
+
+    class Post(ctypes.Structure):
+        _fields_ = [("w", ctypes.c_void_p), ("u", ctypes.c_void_p), ("numel", ctypes.c_int64),
+                    ("lr_ratio", ctypes.c_float), ("w_dtype", ctypes.c_int32)]
+
+    for cs, nd in ((Pre, _lib.PRE_ITEM), (Post, _lib.POST_ITEM)):
+        assert ctypes.sizeof(cs) == nd.itemsize
+        for name, _ in cs._fields_:
+            assert getattr(cs, name).offset == nd.fields[name][1]
+
+
+def test_workspace_and_flops_queries_need_no_gpu():
+    from archscale_amd import _lib
+    L = _lib.lib()
+    assert L.muon_ns_workspace_bytes(0, 8, 8, 0) == 0
+    small = L.muon_ns_workspace_bytes(1, 512, 2048, 0)
+    split = L.muon_ns_workspace_bytes(1, 512, 2048, 1)
+    assert split - small >= 512 * 512 * 2 and small >= 4 * 512 * 2048 * 2 + 2 * 512 * 512 * 2
+    assert L.muon_ns_workspace_bytes(1, 2048, 512, 0) == small            # orientation does not matter
+    d, s, i = _lib.ns_flops(1, 512, 2048, 5, 0)
+    assert d == pytest.approx(5 * (4 * 512 ** 2 * 2048 + 2 * 512 ** 3))
+    assert s == pytest.approx(5 * (3 * 512 ** 2 * 2048 + 512 ** 3))
+    assert s < i < d                                                        # full diagonal tiles cost a little
+    d2, s2, i2 = _lib.ns_flops(1, 512, 2048, 5, 1)
+    assert i2 > i and d2 == d
+    assert L.muon_muonh_scratch_floats(3, 10) >= 3 * 10 + 2 * 3
+
+
+def test_argument_errors_without_touching_the_gpu():
+    from archscale_amd import _lib
+    L = _lib.lib()
+    abc = _lib.abc_array([(1.0, 0.0, 0.0)])
+    assert L.muon_ns_batched(None, 0, 0, 8, None, 0, 8, 1, 8, 8, abc, 1, 1e-7, 0, 0, 0, None, 0, None) == -1
+    assert L.muon_momentum(None, None, 3, 3, 0.9, 1.0, 0.9, 1.0, 0.0, None) == -1
+    assert L.muon_momentum(None, None, 0, 0, 0.9, 1.0, 0.9, 1.0, 0.0, None) == 0   # nothing to do
+    assert L.muon_update_muonh(None, None, 2, 2, 0.1, 0.0, 1e-8, 0, None, None) == -1
+    with pytest.raises(ValueError):
+        _lib.check(-1, "x")
+    with pytest.raises(_lib.MuonLibraryError):
+        _lib.check(1, "x")
+    with pytest.raises(TypeError):
+        _lib.dtype_code(torch.float16)
+
+
+def test_no_cpu_fallback():
+    import archscale_amd.optim.newton_schulz_hip as H
+    from archscale_amd._lib import MuonLibraryError
+    from archscale_amd.optim.muon import Muon
+    with pytest.raises(MuonLibraryError):
+        H.zeropower_via_newtonschulz5(torch.randn(8, 16))
+    p = torch.nn.Parameter(torch.randn(8, 16))
+    p.grad = torch.randn(8, 16)
+    opt = Muon([p])
+    with pytest.raises(MuonLibraryError):
+        opt.step()
+    assert opt.param_groups[0]["step"] == 1   # counted before the work, as in the reference
+
+
+def test_constructor_validation_and_defaults():
+    from archscale_amd.optim.muon import Muon
+    p = torch.nn.Parameter(torch.randn(4, 4))
+    for bad in (dict(lr=-1.0), dict(mu=-0.1), dict(betas=(0.9,)), dict(betas=(-0.1, 0.9)), dict(adjust_lr="nope")):
+        with pytest.raises(ValueError):
+            Muon([p], **bad)
+    with pytest.raises(TypeError):
+        Muon([p], distributed_mesh="mesh")
+    with pytest.raises(TypeError):
+        Muon([p], newton_schulz_func=3)
+    opt = Muon([p], betas=(0.8, 0.9), use_triton=True)
+    g = opt.param_groups[0]
+    assert (g["lr"], g["mu"], g["beta1"], g["beta2"], g["weight_decay"], g["epsilon"]) == (0.01, 0.95, 0.8, 0.9, 0.01, 1e-8)
+    assert g["algorithm"] == "muon" and g["step"] == 0 and g["nesterov"] is False and g["flatten"] is False
+    assert g["adjust_lr"] == "spectral_norm" and g["cautious_wd"] is False
+    assert opt.use_muonh is False and opt._world_size == 1
+    opt.exclude_from_hyperball(p)
+    assert p in opt._hyperball_excluded
+    # 1-D parameter in a muon group is refused
+    v = torch.nn.Parameter(torch.randn(4))
+    v.grad = torch.randn(4)
+    with pytest.raises(AssertionError):
+        Muon([v]).step()
+
+
+def test_lr_ratios_flatten_policy_and_batches():
+    from archscale_amd.optim import muon as M
+    from archscale_amd.optim.opt_utils import create_param_batches, matrix_view_shape
+    assert M.adjust_lr_spectral_norm(0.02, (5632, 2048), False) == pytest.approx(0.02 * math.sqrt(2.75))
+    assert M.adjust_lr_spectral_norm(0.02, (2048, 5632), False, clip_norm=True) == pytest.approx(0.02)
+    assert M.adjust_lr_rms_norm(0.02, (64, 512, 2048), False) == pytest.approx(0.02 * 0.2 * math.sqrt(2048))
+    assert M.adjust_lr_spectral_norm(1.0, (64, 8, 4), True) == pytest.approx(math.sqrt(2.0))
+    assert M._lr_ratio((8, 2), None, False) == 1.0
+    with pytest.raises(ValueError):
+        M._lr_ratio((8, 2), "bad", False)
+    assert matrix_view_shape((6, 4), False) == (1, 6, 4)
+    assert matrix_view_shape((3, 6, 4), False) == (3, 6, 4)
+    assert matrix_view_shape((2, 3, 6, 4), False) == (6, 6, 4)
+    assert matrix_view_shape((2, 3, 6, 4), True) == (1, 2, 72)
+    with pytest.raises(ValueError):
+        matrix_view_shape((5,), False)
+    ps = [torch.zeros(2, 3), torch.zeros(3, 2), torch.zeros(2, 3), torch.zeros(2, 3, dtype=torch.bfloat16),
+          torch.zeros(2, 3)]
+    got = [[id(t) for t in b] for b in create_param_batches(ps, 2)]
+    assert got == [[id(ps[0]), id(ps[2])], [id(ps[4])], [id(ps[1])], [id(ps[3])]]
+
+
+def test_emerging_host_logic():
+    from archscale_amd.emerging import get_muon_scale_factor
+    from archscale_amd.emerging.mixin import weight_decay_terms
+    from archscale_amd.emerging.spectral_ball_utils import msign_schedule, MSIGN_COEFFICIENTS
+    from archscale_amd.emerging import Muon as EMuon, newton_schulz, msign
+    assert get_muon_scale_factor(8, 2, "shape_scaling") == 2.0
+    assert get_muon_scale_factor(100, 400, "align_adamw_rms") == pytest.approx(4.0)
+    assert get_muon_scale_factor(8, 2, "spectral_mup") == 2.0
+    with pytest.raises(ValueError):
+        get_muon_scale_factor(1, 1)          # the reference's default "spectral" is not a valid mode either
+    assert weight_decay_terms("decoupled", 0.1, 0.5) == (0.05, 0.0)
+    assert weight_decay_terms("independent", 0.1, 0.5) == (0.5, 0.0)
+    assert weight_decay_terms("l2", 0.1, 0.5) == (0.0, 0.5)
+    assert weight_decay_terms("l2", 0.1, 0.0) == (0.0, 0.0)
+    with pytest.raises(ValueError):
+        weight_decay_terms("bad", 0.1, 0.5)
+    assert msign_schedule(10)[9] == MSIGN_COEFFICIENTS[7] and len(msign_schedule(5)) == 5
+    with pytest.raises(ValueError):
+        EMuon([torch.nn.Parameter(torch.zeros(2, 2))], num_ns_steps=0)
+    with pytest.raises(ValueError):
+        msign(torch.zeros(4, 4, dtype=torch.bfloat16), 5)
+    with pytest.raises(ValueError):
+        newton_schulz(torch.zeros(4, 4), steps=3, coefficient_type="quintic")   # 3 is no multiple of 5
+    with pytest.raises(ValueError):
+        newton_schulz(torch.zeros(4, 4), steps=5, coefficient_type="nope")
+    o = EMuon([torch.nn.Parameter(torch.zeros(2, 2))])
+    g = o.param_groups[0]
+    assert (g["lr"], g["momentum_beta"], g["weight_decay"]) == (3e-4, 0.95, 0.01)
+    assert np.isclose(o._extra_scale_factor, 1.0)

@@ -1,0 +1,286 @@
+"""Parity of the Muon / MuonH optimizer step (HIP, through the C ABI) against the CPU oracle.
+
+Bars (from the path's contract): updated weights within 2e-2 relative error of the reference step.
+Because a MuonH step at lr 0.02 moves the weights by exactly 2e-2, W parity alone cannot see a
+missing update, so every test also checks the weight DELTA (with fp32 weights, where it is meaningful).
+"""
+import copy
+import math
+
+import pytest
+import torch
+
+from oracle import muon_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+W_TOL = 2e-2      # relative Frobenius error on updated weights (contract)
+DW_TOL = 3e-2     # on the weight delta with fp32 weights: NS error (<= 1e-2) plus bf16 rounding of U
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def _make(shapes, dtype, seed, device, gdtype=None):
+    g = torch.Generator().manual_seed(seed)
+    ps = []
+    for s in shapes:
+        w = (torch.randn(*s, generator=g) * 0.02).to(dtype)
+        p = torch.nn.Parameter(w.to(device))
+        ps.append(p)
+    return ps
+
+
+def _grads(shapes, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(*s, generator=g) * 1e-3).to(dtype) for s in shapes]
+
+
+SHAPES = [(128, 256), (256, 128), (128, 256), (64, 64), (3, 64, 192), (2, 192, 64)]
+
+
+def _oracle_run(shapes, w0, grads_per_step, *, wdtype, hp, use_muonh, ns_storage, per_matrix=False):
+    X = [w.clone().to(wdtype) for w in w0]
+    M = [torch.zeros_like(x) for x in X]
+    for grads in grads_per_step:
+        for x, g, m in zip(X, grads, M):
+            if use_muonh and per_matrix and x.ndim == 3:
+                # per-matrix renormalisation = the reference applied to each expert as its own parameter
+                U = O.muon_pre_orthogonalize(g, m, hp["mu"], hp["nesterov"])
+                Oo = O.newton_schulz(U, O.QUINTIC, hp["eps"], storage=ns_storage).to(torch.bfloat16)
+                for e in range(x.shape[0]):
+                    O.muonh_post_orthogonalize(x[e], Oo[e], hp["lr"], hp["wd"], hp["eps"], hp["cautious"])
+            else:
+                O.lit_gpt_muon_step(x, g, m, lr=hp["lr"], mu=hp["mu"], wd=hp["wd"], eps=hp["eps"],
+                                    nesterov=hp["nesterov"], adjust=hp["adjust"], flatten=False,
+                                    cautious=hp["cautious"], use_muonh=use_muonh, ns_storage=ns_storage)
+    return X, M
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_muonh", [False, True])
+@pytest.mark.parametrize("wd,cautious", [(0.0, False), (0.1, True)])
+def test_step_matches_oracle(gpu_device, wdtype, use_muonh, wd, cautious):
+    from archscale_amd.optim.muon import Muon
+    hp = dict(lr=0.02, mu=0.95, wd=wd, eps=1e-8, nesterov=True, adjust="spectral_norm", cautious=cautious)
+    params = _make(SHAPES, wdtype, 1, gpu_device)
+    w0 = [p.detach().cpu().clone() for p in params]
+    opt = Muon(params, lr=hp["lr"], mu=hp["mu"], weight_decay=wd, cautious_wd=cautious, epsilon=hp["eps"],
+               nesterov=True, adjust_lr="spectral_norm", use_muonh=use_muonh)
+    steps = [_grads(SHAPES, wdtype, 100 + k) for k in range(3)]
+    for grads in steps:
+        for p, g in zip(params, grads):
+            p.grad = g.to(gpu_device)
+        opt.step()
+    torch.cuda.synchronize()
+    # reference semantics, bf16 eager NS (what the reference's CPU path computes)
+    Xr, Mr = _oracle_run(SHAPES, w0, steps, wdtype=wdtype, hp=hp, use_muonh=use_muonh, ns_storage="bf16_eager")
+    # the same step with the tolerance oracle for NS (fp32 on the same bf16 inputs)
+    Xf, _ = _oracle_run(SHAPES, w0, steps, wdtype=wdtype, hp=hp, use_muonh=use_muonh, ns_storage="fp32")
+    for p, xr, xf, w, mr in zip(params, Xr, Xf, w0, Mr):
+        assert _rel(p.detach(), xr) <= W_TOL
+        assert _rel(p.detach(), xf) <= W_TOL
+        m = opt.state[p]["momentum"]
+        assert m.dtype == p.dtype and _rel(m, mr) <= (1e-6 if wdtype == torch.float32 else 1e-2)
+        if wdtype == torch.float32:
+            dw, dwf = p.detach().cpu() - w, xf - w
+            assert _rel(dw, dwf) <= DW_TOL
+            if use_muonh:
+                # norm preservation (after the decay, which is the only thing allowed to change the norm)
+                assert p.detach().norm().item() == pytest.approx(xf.norm().item(), rel=1e-4)
+    for g in opt.param_groups:
+        assert g["step"] == 3
+
+
+def test_muonh_per_matrix_and_whole_tensor(gpu_device):
+    """A 3-D expert stack: the default renormalises the whole tensor (what the reference does for one
+    3-D Parameter), ``muonh_per_matrix`` renormalises each expert."""
+    from archscale_amd.optim.muon import Muon
+    shapes = [(8, 64, 128), (8, 128, 32)]
+    hp = dict(lr=0.05, mu=0.95, wd=0.0, eps=1e-8, nesterov=True, adjust="spectral_norm", cautious=False)
+    grads = [_grads(shapes, torch.float32, 7)]
+    for per_matrix in (False, True):
+        params = _make(shapes, torch.float32, 2, gpu_device)
+        # give the experts different scales so that the two conventions differ visibly
+        with torch.no_grad():
+            for p in params:
+                p.mul_(torch.linspace(0.5, 2.0, 8, device=gpu_device).view(8, 1, 1))
+        w0 = [p.detach().cpu().clone() for p in params]
+        opt = Muon(params, lr=hp["lr"], mu=hp["mu"], weight_decay=0.0, nesterov=True, use_muonh=True,
+                   muonh_per_matrix=per_matrix)
+        for p, g in zip(params, grads[0]):
+            p.grad = g.to(gpu_device)
+        opt.step()
+        Xf, _ = _oracle_run(shapes, w0, grads, wdtype=torch.float32, hp=hp, use_muonh=True, ns_storage="fp32",
+                            per_matrix=per_matrix)
+        for p, xf, w in zip(params, Xf, w0):
+            assert _rel(p.detach().cpu() - w, xf - w) <= DW_TOL
+            if per_matrix:
+                for e in range(8):
+                    assert p[e].norm().item() == pytest.approx(w[e].norm().item(), rel=1e-4)
+            else:
+                assert p.norm().item() == pytest.approx(w.norm().item(), rel=1e-4)
+                assert max(abs(p[e].norm().item() / w[e].norm().item() - 1) for e in range(8)) > 1e-4
+
+
+def test_batched_equals_one_by_one(gpu_device):
+    """Shape-class batching must not change any tensor's result: one optimizer over all parameters
+    equals one optimizer per parameter, bit for bit."""
+    from archscale_amd.optim.muon import Muon
+    grads = _grads(SHAPES, torch.bfloat16, 9)
+    pa = _make(SHAPES, torch.bfloat16, 3, gpu_device)
+    pb = _make(SHAPES, torch.bfloat16, 3, gpu_device)
+    kw = dict(lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0)
+    oa = Muon(pa, **kw)
+    obs = [Muon([p], **kw) for p in pb]
+    for _ in range(2):
+        for p, q, g in zip(pa, pb, grads):
+            p.grad = g.to(gpu_device)
+            q.grad = g.to(gpu_device)
+        oa.step()
+        for o in obs:
+            o.step()
+    for p, q in zip(pa, pb):
+        assert torch.equal(p, q)
+
+
+def test_hook_state_dict_and_groups(gpu_device):
+    from archscale_amd.optim.muon import Muon
+    import archscale_amd.optim.newton_schulz_hip as H
+    shapes = [(64, 128), (128, 64)]
+    params = _make(shapes, torch.float32, 4, gpu_device)
+    vec = torch.nn.Parameter(torch.randn(128, device=gpu_device))
+    emb = torch.nn.Parameter(torch.randn(50, 64, device=gpu_device))
+    head = torch.nn.Parameter(torch.randn(50, 64, device=gpu_device))
+    calls = []
+
+    def hook(X, epsilon):
+        calls.append((tuple(X.shape), float(epsilon)))
+        return H.newton_schulz_hip(X, epsilon)
+
+    lion_vec = torch.nn.Parameter(torch.randn(32, device=gpu_device))
+    groups = [dict(params=params), dict(params=[vec, emb, head], algorithm="adamw", lr=1e-3),
+              dict(params=[lion_vec], algorithm="lion", lr=1e-3)]
+    opt = Muon(groups, lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0, newton_schulz_func=hook)
+    opt.exclude_from_hyperball(emb)
+    ref = Muon(copy.deepcopy(groups), lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0)
+    for p, q in zip(opt.param_groups[0]["params"], ref.param_groups[0]["params"]):
+        g = torch.randn_like(p) * 1e-3
+        p.grad, q.grad = g, g.clone()
+    for p, q in zip(opt.param_groups[1]["params"], ref.param_groups[1]["params"]):
+        g = torch.randn_like(p) * 1e-2
+        p.grad, q.grad = g, g.clone()
+    emb_norm, head_norm = emb.norm().item(), head.norm().item()
+    opt.step()
+    ref.step()
+    assert sorted(calls) == sorted([((64, 128), 1e-8), ((128, 64), 1e-8)]) or len(calls) == 2
+    for p, q in zip(opt.param_groups[0]["params"], ref.param_groups[0]["params"]):
+        assert torch.equal(p, q)  # the hook runs the same kernels as the built-in path
+    # hyperball AdamW keeps the norm of 2-D non-excluded tensors only
+    assert head.norm().item() == pytest.approx(head_norm, rel=1e-5)
+    assert abs(emb.norm().item() / emb_norm - 1) > 1e-6
+    # state dict round trip
+    sd = opt.state_dict()
+    assert all("momentum" in s for s in sd["state"].values())
+    assert sd["param_groups"][0]["step"] == 1 and sd["param_groups"][1]["algorithm"] == "adamw"
+    opt2 = Muon(groups, lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0)
+    opt2.load_state_dict(sd)
+    assert opt2.param_groups[0]["step"] == 1
+    for p in params:
+        assert torch.equal(opt2.state[p]["momentum"], opt.state[p]["momentum"])
+    # closure and unknown algorithm
+    assert opt.step(lambda: torch.tensor(3.0)).item() == 3.0
+    opt.param_groups[2]["algorithm"] = "sgd"
+    with pytest.raises(ValueError):
+        opt.step()
+
+
+def test_first_step_and_missing_grads(gpu_device):
+    from archscale_amd.optim.muon import Muon
+    import archscale_amd.optim.newton_schulz_hip as H
+    params = _make([(64, 128), (64, 128)], torch.float32, 5, gpu_device)
+    w0 = [p.detach().clone() for p in params]
+    opt = Muon(params, lr=0.1, mu=0.9, nesterov=True, weight_decay=0.0, adjust_lr=None)
+    g = (torch.randn(64, 128, device=gpu_device) * 1e-3)
+    params[0].grad = g
+    opt.step()                       # params[1] has no grad: untouched, no state
+    assert torch.equal(params[1], w0[1]) and len(opt.state[params[1]]) == 0
+    # from zero momentum U = (1+mu) G, so the update is lr * NS(bf16((1+mu) G))
+    ns_out = H.newton_schulz_hip(((1.9 * g)).to(torch.bfloat16), 1e-8).float()
+    assert _rel(params[0].detach() - w0[0], -0.1 * ns_out) < 1e-2
+    assert torch.allclose(opt.state[params[0]]["momentum"], g)
+
+
+def test_emerging_muon_matches_oracle(gpu_device):
+    from archscale_amd.emerging import Muon as EMuon
+    shapes = [(64, 128), (128, 64), (64, 128)]
+    for method, nesterov in (("decoupled", True), ("independent", False), ("l2", True)):
+        params = _make(shapes, torch.float32, 6, gpu_device)
+        w0 = [p.detach().cpu().clone() for p in params]
+        opt = EMuon(params, lr=0.01, momentum_beta=0.9, weight_decay=0.1, use_nesterov=nesterov,
+                    weight_decay_method=method, scale_mode="spectral_mup", extra_scale_factor=1.5)
+        steps = [_grads(shapes, torch.float32, 40 + k) for k in range(2)]
+        X = [w.clone() for w in w0]
+        B = [torch.zeros_like(w) for w in w0]
+        for grads in steps:
+            for p, g in zip(params, grads):
+                p.grad = g.clone().to(gpu_device)
+            opt.step()
+            for x, g, b in zip(X, grads, B):
+                O.emerging_muon_step(x, g.clone(), b, lr=0.01, beta=0.9, wd=0.1, nesterov=nesterov,
+                                     wd_method=method, steps=5, scale_mode="spectral_mup", extra_scale=1.5,
+                                     ns_storage="fp32")
+        for p, x, w, b in zip(params, X, w0, B):
+            assert _rel(p.detach(), x) <= W_TOL
+            assert _rel(p.detach().cpu() - w, x - w) <= DW_TOL
+            assert _rel(opt.state[p]["momentum_buffer"], b) <= 1e-5
+    with pytest.raises(ValueError):
+        o = EMuon([torch.nn.Parameter(torch.randn(8, device=gpu_device))])
+        o.param_groups[0]["params"][0].grad = torch.randn(8, device=gpu_device)
+        o.step()
+
+
+def test_emerging_hook_path(gpu_device):
+    from archscale_amd.emerging import OrthogonalizedOptimizer, msign
+    p = torch.nn.Parameter((torch.randn(64, 96) * 0.02).to(gpu_device))
+    p.param_name = "blk.w"
+    w0 = p.detach().clone()
+    opt = OrthogonalizedOptimizer([p], 0.1, 0.9, 0.0, use_nesterov=False, weight_decay_method="decoupled",
+                                  fp32_matmul_prec="medium", scaled_orthogonalize_fn=lambda g: msign(g, 5),
+                                  log_per_module_update_rms=True, log_per_module_grad_rms=True)
+    g = torch.randn(64, 96, device=gpu_device) * 1e-3
+    p.grad = g
+    opt.step()
+    want = msign(0.1 * g, 5).float()
+    assert _rel(p.detach() - w0, -0.1 * want) < 1e-2
+    assert opt.get_update_rms_dict()["blk.w"] == pytest.approx(math.sqrt(1 / 96), rel=0.2)
+    assert opt.get_grad_rms_dict()["blk.w"] == pytest.approx((0.1 * g).pow(2).mean().sqrt().item(), rel=1e-3)
+
+
+def test_config3_expert_batches(gpu_device):
+    """64 experts, W1/W3 stacked 512x2048 and W2 2048x256 (tall => transposed), one batched launch per
+    kernel, per-expert MuonH renormalisation; checked on a seeded subset of experts against the oracle."""
+    from archscale_amd.optim.muon import Muon
+    shapes = [(64, 512, 2048), (64, 2048, 256)]
+    g = torch.Generator().manual_seed(1237)
+    W = [(torch.randn(*s, generator=g) * 0.02).to(torch.bfloat16) for s in shapes]
+    G = [(torch.randn(*s, generator=g) * 1e-3).to(torch.bfloat16) for s in shapes]
+    params = [torch.nn.Parameter(w.to(gpu_device)) for w in W]
+    opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.0, use_muonh=True, muonh_per_matrix=True)
+    for p, gr in zip(params, G):
+        p.grad = gr.to(gpu_device)
+    opt.step()
+    torch.cuda.synchronize()
+    for p, w, gr in zip(params, W, G):
+        for e in (0, 17, 63):
+            x = w[e].clone()
+            m = torch.zeros_like(x)
+            O.lit_gpt_muon_step(x, gr[e], m, lr=0.02, mu=0.95, wd=0.0, eps=1e-8, nesterov=True,
+                                adjust="spectral_norm", flatten=False, cautious=False, use_muonh=True,
+                                ns_storage="bf16_eager")
+            assert _rel(p[e].detach(), x) <= W_TOL
+            # the update is really there: distance to the OLD weights is ~lr, to the new ones much less
+            assert _rel(p[e].detach(), x) < 0.25 * _rel(w[e], x)
+            assert p[e].float().norm().item() == pytest.approx(w[e].float().norm().item(), rel=2e-3)
