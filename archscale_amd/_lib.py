@@ -191,6 +191,6 @@ def profile_collect(capacity: int = 4096):
     out = []
     for i in range(min(n, capacity)):
         k = key[i]
-        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool(k & 2), final=bool(k & 1),
+        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool((k % 10) & 2), final=bool((k % 10) & 1),
                         flops_algorithmic=fa[i], flops_issued=fi[i]))
     return out
