@@ -148,126 +148,210 @@ ns_gemm_kernel(const GemmParams p) {
     rdQ[kk] = lds_chunk_off(wc0 + l32, 2 * kk + hi);
   }
 
+  // Operand fragments are double-buffered in registers: while the MFMAs of k-step kk run, the LDS reads of
+  // kk+1 are issued, one read slotted after each MFMA (the scheduler is pinned to that order below;
+  // left alone it serialises read -> wait -> MFMA and the matrix pipe idles on LDS latency).
+  bf16x8 af[2][FM], bq[2][FN];
+  auto load_frags = [&](int buf, const char* sP, const char* sQ, int kk) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i) af[buf][i] = *(const bf16x8*)(sP + rdP[kk] + i * 32 * ROW_BYTES);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) bq[buf][j] = *(const bf16x8*)(sQ + rdQ[kk] + j * 32 * ROW_BYTES);
+  };
+
   issue(0, 0);
   for (int kt = 0; kt < KT_ALL; ++kt) {
     const int stage = kt & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for `stage` have landed
-    __syncthreads();                             // everyone's have; everyone is done reading the other stage
+    __syncthreads();                                  // everyone's have; everyone is done reading the other stage
     if (kt + 1 < KT_ALL) issue(kt + 1, stage ^ 1);
     const char* sP = smem + stage * STAGE;
     const char* sQ = sP + PBYTES;
+    load_frags(0, sP, sQ, 0);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      bf16x8 af[FM], bq[FN];
-#pragma unroll
-      for (int i = 0; i < FM; ++i) af[i] = *(const bf16x8*)(sP + rdP[kk] + i * 32 * ROW_BYTES);
-#pragma unroll
-      for (int j = 0; j < FN; ++j) bq[j] = *(const bf16x8*)(sQ + rdQ[kk] + j * 32 * ROW_BYTES);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk + 1 < 4) load_frags((kk + 1) & 1, sP, sQ, kk + 1);
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bq[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bq[kk & 1][j], acc[i][j], 0, 0, 0);
+      if (kk + 1 < 4) {
+#pragma unroll
+        for (int q = 0; q < FM + FN; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        }
+        if (FM * FN > FM + FN) __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
   // ---- epilogue.  acc[i][j][e] of lane l is element
-  //   row = R0 + wr0 + i*32 + 8*(e/4) + 4*(l/32) + e%4,   col = C0 + wc0 + j*32 + l%32
-  // so each lane owns 4 consecutive rows of one column: the TRANSPOSED image is an 8-byte store.
+  //   rl = wr0 + i*32 + 8*(e/4) + 4*(l/32) + e%4  (row in the tile),   cl = wc0 + j*32 + l%32  (column)
+  // so a lane owns 4 consecutive rows of one column.  Every global access of the epilogue goes through
+  // LDS (the operand stages are dead by now) so that it is a 16-byte, row-contiguous access:
+  //   * the addend tile is copied in as its transposed image  S[cl][rl]  (it is read as E[col][row..row+3]);
+  //   * the transposed output (mirror of a symmetric product, X'^T) is staged as S[cl][rl] with 8-byte
+  //     LDS writes and flushed row by row;
+  //   * the row-major output is staged as D[rl][cl] with 2-byte LDS writes and flushed row by row.
+  // Scattered 8-byte / 2-byte global accesses straight from the accumulator layout flood L2 with
+  // partial-line requests and cost a quarter of the kernel.
+  static_assert(BM == BN, "square block tiles");
+  constexpr int NT = NW * 64;
+  constexpr int TPITCH = BN * 2;            // bytes per staged row (both images)
+  constexpr int CPRT = BN / 8;              // 16-byte chunks per staged row
+  constexpr int PASSES = (BM * BN / 8) / NT;
+  static_assert(BM * BN * 2 <= 2 * STAGE, "staging tile must fit in the operand stages");
   const float alpha = p.alpha, beta = p.beta;
   const bool diag = SYM && (ti == tj);
+  // S[cl][rl]: chunk index XOR cl, so the 32 lanes of an 8-byte access (32 different cl) spread over all banks
+  auto s_off = [](int cl, int rl) { return cl * TPITCH + ((((rl >> 3) ^ cl) & (CPRT - 1)) << 4) + ((rl & 7) << 1); };
+  auto s_chunk = [](int cl, int ch) { return cl * TPITCH + (((ch ^ cl) & (CPRT - 1)) << 4); };
+  // D[rl][cl]: 64-byte halves of a row swapped on rows with bit 2 set, so the two half-waves of a 2-byte
+  // access (rows r and r+4) hit different banks
+  auto d_off = [](int rl, int byte_in_row) { return rl * TPITCH + (byte_in_row ^ (((rl >> 2) & 1) << 6)); };
+
+  // row-contiguous copy of a staged image to global memory; `swz` maps (staged row, chunk) -> LDS offset
+  auto flush = [&](auto swz, __bf16* dst, long bstride, int ld, int row0, int col0, int rows_valid, int cols_valid) {
+    __bf16* base = dst + (size_t)b * bstride;
+    const bool vec_ok = !FINAL || ((ld & 7) == 0 && (bstride & 7) == 0 && (((uintptr_t)dst) & 15) == 0);
+#pragma unroll 4
+    for (int t = 0; t < PASSES; ++t) {
+      const int q = t * NT + tid;
+      const int sr = q / CPRT, ch = q - sr * CPRT;
+      const uint4 val = *(const uint4*)(smem + swz(sr, ch));
+      const int row = row0 + sr, col = col0 + ch * 8;
+      if (!FINAL) {
+        *(uint4*)(base + (size_t)row * ld + col) = val;
+      } else if (row < rows_valid) {  // caller's tensor: true extents, arbitrary leading dimension
+        if (vec_ok && col + 7 < cols_valid) {
+          *(uint4*)(base + (size_t)row * ld + col) = val;
+        } else {
+          const uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
+          for (int k = 0; k < 8; ++k)
+            if (col + k < cols_valid) ((uint16_t*)base)[(size_t)row * ld + col + k] = (uint16_t)(w[k >> 1] >> ((k & 1) * 16));
+        }
+      }
+    }
+  };
+  auto s_swz = [&](int sr, int ch) { return s_chunk(sr, ch); };
+  auto d_swz = [&](int sr, int ch) { return d_off(sr, ch * 16); };
+
+  __syncthreads();  // every wave is done reading the operand stages
+
+  // 1. fold the addend into the accumulators: acc <- alpha*acc + beta*E (SYRK2), acc + alpha*E (BX), alpha*acc (SYRK)
+  if (MODE != MODE_SYRK) {
+    // E[C0 + cl][R0 + rl] -> S[cl][rl], two staged rows (1 KiB) per wave-wide copy
+    const char* Eb = (const char*)(p.E + (size_t)b * p.strideE + (size_t)C0 * p.lde + R0);
+#pragma unroll
+    for (int t = 0; t < PASSES; ++t) {
+      const int slab = wave * PASSES + t;                  // 64 chunks
+      const int q = slab * 64 + lane;
+      const int sr = q / CPRT, cpos = q - sr * CPRT;
+      const int src = (cpos ^ sr) & (CPRT - 1);
+      __builtin_amdgcn_global_load_lds((gptr_t)(Eb + ((size_t)sr * p.lde + src * 8) * 2), (lptr_t)(smem + slab * 1024), 16, 0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
-      const int col = C0 + wc0 + j * 32 + l32;
+      const int cl = wc0 + j * 32 + l32;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int row = R0 + wr0 + i * 32 + 8 * g + 4 * hi;
-        float v[4];
+        const int rl = wr0 + i * 32 + 8 * g + 4 * hi;
+        if (MODE == MODE_SYRK) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = acc[i][j][4 * g + q];
-
-        if (MODE == MODE_SYRK || MODE == MODE_SYRK2) {
-          __bf16* C = p.C + (size_t)b * p.strideC;
-          __bf16* C2 = SPLIT ? p.C2 + (size_t)b * p.strideC : nullptr;
-          float lo[4];
+          for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
+        } else {
+          const uint2 e = *(const uint2*)(smem + s_off(cl, rl));
+          const float e0 = bf16_to_f32(e.x & 0xffff), e1 = bf16_to_f32(e.x >> 16);
+          const float e2 = bf16_to_f32(e.y & 0xffff), e3 = bf16_to_f32(e.y >> 16);
           if (MODE == MODE_SYRK2) {
-            // addend A[row+q][col] == A[col][row+q] (A is stored exactly symmetric)
-            const uint2 e = *(const uint2*)(p.E + (size_t)b * p.strideE + (size_t)col * p.lde + row);
-            const float a0 = bf16_to_f32(e.x & 0xffff), a1 = bf16_to_f32(e.x >> 16);
-            const float a2 = bf16_to_f32(e.y & 0xffff), a3 = bf16_to_f32(e.y >> 16);
-            v[0] = alpha * v[0] + beta * a0;
-            v[1] = alpha * v[1] + beta * a1;
-            v[2] = alpha * v[2] + beta * a2;
-            v[3] = alpha * v[3] + beta * a3;
+            acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
+            acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
+            acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
+            acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
           } else {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] *= alpha;
-          }
-          if (SPLIT) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) lo[q] = v[q] - bf16_to_f32(bf16_bits(v[q]));
-          }
-          if (!diag) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              ((uint16_t*)C)[(size_t)(row + q) * p.ldc + col] = bf16_bits(v[q]);
-              if (SPLIT) ((uint16_t*)C2)[(size_t)(row + q) * p.ldc + col] = bf16_bits(lo[q]);
-            }
-            *(uint2*)(C + (size_t)col * p.ldc + row) = pack4(v[0], v[1], v[2], v[3]);
-            if (SPLIT) *(uint2*)(C2 + (size_t)col * p.ldc + row) = pack4(lo[0], lo[1], lo[2], lo[3]);
-          } else {
-            // diagonal tile: keep the upper half and reflect it, so the result is bit-symmetric
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              if (col >= row + q) {
-                ((uint16_t*)C)[(size_t)(row + q) * p.ldc + col] = bf16_bits(v[q]);
-                ((uint16_t*)C)[(size_t)col * p.ldc + row + q] = bf16_bits(v[q]);
-                if (SPLIT) {
-                  ((uint16_t*)C2)[(size_t)(row + q) * p.ldc + col] = bf16_bits(lo[q]);
-                  ((uint16_t*)C2)[(size_t)col * p.ldc + row + q] = bf16_bits(lo[q]);
-                }
-              }
-            }
-          }
-        } else {  // MODE_BX: v = acc + alpha * X[row+q][col], X[row+q][col] == Xt[col][row+q]
-          const uint2 e = *(const uint2*)(p.E + (size_t)b * p.strideE + (size_t)col * p.lde + row);
-          v[0] += alpha * bf16_to_f32(e.x & 0xffff);
-          v[1] += alpha * bf16_to_f32(e.x >> 16);
-          v[2] += alpha * bf16_to_f32(e.y & 0xffff);
-          v[3] += alpha * bf16_to_f32(e.y >> 16);
-          if (!FINAL) {
-            if (p.C) {
-              uint16_t* C = (uint16_t*)(p.C + (size_t)b * p.strideC);
-#pragma unroll
-              for (int q = 0; q < 4; ++q) C[(size_t)(row + q) * p.ldc + col] = bf16_bits(v[q]);
-            }
-            if (p.Ct) *(uint2*)(p.Ct + (size_t)b * p.strideCt + (size_t)col * p.ldct + row) = pack4(v[0], v[1], v[2], v[3]);
-          } else {
-            // caller's tensor: true extents, arbitrary leading dimension
-            if (p.C) {
-              uint16_t* C = (uint16_t*)(p.C + (size_t)b * p.strideC);
-              if (col < p.n_valid) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                  if (row + q < p.m_valid) C[(size_t)(row + q) * p.ldc + col] = bf16_bits(v[q]);
-              }
-            }
-            if (p.Ct && col < p.n_valid) {
-              __bf16* Ct = p.Ct + (size_t)b * p.strideCt + (size_t)col * p.ldct + row;
-              if (row + 3 < p.m_valid && (p.ldct & 3) == 0 && (p.strideCt & 3) == 0) {
-                *(uint2*)Ct = pack4(v[0], v[1], v[2], v[3]);
-              } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                  if (row + q < p.m_valid) ((uint16_t*)Ct)[q] = bf16_bits(v[q]);
-              }
-            }
+            acc[i][j][4 * g + 0] += alpha * e0;
+            acc[i][j][4 * g + 1] += alpha * e1;
+            acc[i][j][4 * g + 2] += alpha * e2;
+            acc[i][j][4 * g + 3] += alpha * e3;
           }
         }
       }
     }
+  if (MODE != MODE_SYRK) __syncthreads();  // the addend image is consumed; LDS is free again
+
+  // stores the accumulators as bf16 to Cdst (row-major image) and to its transposed / mirrored image
+  auto store_all = [&](__bf16* Cdst) {
+    // 2. transposed image
+    const bool want_t = SYM ? !diag : (p.Ct != nullptr);
+    if (want_t) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int cl = wc0 + j * 32 + l32;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int rl = wr0 + i * 32 + 8 * g + 4 * hi;
+            *(uint2*)(smem + s_off(cl, rl)) =
+                pack4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+          }
+        }
+      __syncthreads();
+      if (SYM) flush(s_swz, Cdst, p.strideC, p.ldc, C0, R0, 0, 0);
+      else flush(s_swz, p.Ct, p.strideCt, p.ldct, C0, R0, p.n_valid, p.m_valid);
+      __syncthreads();
+    }
+    // 3. row-major image
+    if (SYM || p.C) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int cl = wc0 + j * 32 + l32;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int rl = wr0 + i * 32 + 8 * g + 4 * hi + q;
+              const uint16_t bits = bf16_bits(acc[i][j][4 * g + q]);
+              if (!diag) {
+                *(uint16_t*)(smem + d_off(rl, cl * 2)) = bits;
+              } else if (cl >= rl) {
+                // diagonal tile: keep the upper half and reflect it, so the product is bit-symmetric
+                *(uint16_t*)(smem + d_off(rl, cl * 2)) = bits;
+                *(uint16_t*)(smem + d_off(cl, rl * 2)) = bits;
+              }
+            }
+          }
+        }
+      __syncthreads();
+      flush(d_swz, Cdst, p.strideC, p.ldc, R0, C0, p.m_valid, p.n_valid);
+    }
+  };
+
+  store_all(p.C);
+  if (SPLIT && MODE == MODE_SYRK2) {
+    __builtin_amdgcn_sched_barrier(0);
+    // low half of the bf16 split: acc <- acc - bf16(acc), stored the same way to C2
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] -= bf16_to_f32(bf16_bits(acc[i][j][e]));
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    store_all(p.C2);
   }
 }
 
