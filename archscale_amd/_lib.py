@@ -53,6 +53,7 @@ _SIGNATURES = {
     "muon_profile_collect": (ctypes.c_int, [
         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_double),
         ctypes.POINTER(ctypes.c_double), ctypes.c_int]),
+    "muon_calibration_copy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_syrk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
     "muon_syrk": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,

@@ -250,6 +250,11 @@ int muon_syrk(const void* a_dev, int64_t a_batch_stride, int lda, const void* c_
   return (int)launch_unpad_copy(Dp, (long)Np * Np, Np, d_dev, d_batch_stride, ldd, batch, n, n, stream);
 }
 
+int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {
+  if (!src_dev || !dst_dev || (bytes & 15) || ((uintptr_t)src_dev & 15) || ((uintptr_t)dst_dev & 15)) return MUON_E_ARG;
+  return (int)launch_calibration_copy(src_dev, dst_dev, bytes, (hipStream_t)stream);
+}
+
 int muon_profile_begin(void) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   for (auto& r : g_prof) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }

@@ -40,4 +40,6 @@ hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n
 hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
                              float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream);
 
+hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+
 }  // namespace archscale

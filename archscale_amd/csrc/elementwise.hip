@@ -497,4 +497,23 @@ hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// plain copy of known size: calibrates the HBM byte counters (FETCH_SIZE / WRITE_SIZE) of a profiling run
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+calibration_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long n16) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
+  const long n16 = (long)(bytes / 16);
+  if (n16 <= 0) return hipSuccess;
+  long blocks = (n16 + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(calibration_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint4*)src,
+                     (uint4*)dst, n16);
+  return hipGetLastError();
+}
+
 }  // namespace archscale

@@ -85,6 +85,20 @@ def cpu_baseline(coeffs_name, seed, budget_s=15.0):
     }
 
 
+def measured_traffic(kernel_name):
+    """HBM bytes per launch of `kernel_name` from the committed counter summary (two `rocprofv3 --pmc` runs,
+    FETCH_SIZE and WRITE_SIZE, each scaled by the reading of a plain copy of known size), or None."""
+    path = os.path.join(ROOT, "profiles", "bench_config2_ns_gemm_and_epilogues.md")
+    try:
+        for line in open(path):
+            line = line.strip()
+            if line.startswith("traffic_bytes_per_launch") and kernel_name in line:
+                return float(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +109,8 @@ def main():
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="(debug) fewer layers; the result is then not the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=1236)
+    ap.add_argument("--calibration-copy-mib", type=int, default=1024,
+                    help="size of the plain device copy run once after the steps (yardstick for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every box here has one); --gpus must be 1")
@@ -136,6 +152,17 @@ def main():
         phases[name] = phases.get(name, 0.0) + a.elapsed_time(b)
     opt.phase_events = None
 
+    # one plain copy of known size: `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` readings are scaled by what the same
+    # counter reports for this dispatch (calibration_copy_kernel)
+    cal_bytes = args.calibration_copy_mib << 20
+    if cal_bytes:
+        src = torch.empty(cal_bytes, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        _lib.check(_lib.lib().muon_calibration_copy(src.data_ptr(), dst.data_ptr(), cal_bytes,
+                                                    _lib.current_stream_ptr(dev)), "muon_calibration_copy")
+        torch.cuda.synchronize()
+        del src, dst
+
     shapes = [tuple(p.shape) for p in params]
     n_elem = sum(p.numel() for p in params)
     f_dense = sum(dense_flops(s) for s in shapes)
@@ -163,10 +190,16 @@ def main():
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
         "kernel": f"ns_gemm_kernel<{dom_key[0]},{names[dom_key[1]]}{',split' if dom_key[2] else ''}"
                   f"{',final' if dom_key[3] else ''}>",
+        "algorithmic_bytes_per_launch": None,
         "launches": dom["n"], "avg_launch_ms": round(dom["ms"] / dom["n"], 4),
         "flops_per_launch": dom["fa"] / dom["n"],
         "issued_frac": round(dom["fi"] / dom["ms"] / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
     }
+    if args.layers == N_LAYERS:
+        roofline["traffic"] = measured_traffic(roofline["kernel"])
+    if dom_key[1] == 2:  # B (m^2), X^T read twice (operand + addend), X' and X'^T written: bf16
+        per = [(min(s) ** 2 + 4 * min(s) * max(s)) * 2.0 for s in shapes]
+        roofline["algorithmic_bytes_per_launch"] = sum(per) * (4 if not dom_key[3] else 1) / 5 / dom["n"]
     gemm_ms = sum(d["ms"] for d in by_kernel.values())
     f_issued = sum(d["fi"] for d in by_kernel.values())
     hbm = {}
@@ -198,6 +231,7 @@ def main():
         "kernels": kernels,
         "hbm_kernels": hbm,
         "phases_ms": {k: round(v, 3) for k, v in phases.items()},
+        "calibration_copy_bytes": cal_bytes,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.coeffs, args.seed)

@@ -91,6 +91,10 @@ int muon_profile_begin(void);
 int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algorithmic_host,
                          double* flops_issued_host, int capacity);
 
+/* dst <- src, `bytes` (multiple of 16) of device memory with one plain copy kernel.  No counterpart in the
+ * reference: a copy of known size is the yardstick that scales the HBM byte counters of a profiling run. */
+int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream);
+
 /* ---- single products on caller tensors ------------------------------------------------------
  * D = alpha * A A^T + beta * C, A [batch] n x k (bf16, row-major, ld lda), C symmetric n x n or NULL, D n x n,
  * both triangles written.  Replaces ns_line_1 / ns_line_2 (newton_schulz_triton.py:142-178, 269-310) and
