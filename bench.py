@@ -199,7 +199,7 @@ def main():
         roofline["traffic"] = measured_traffic(roofline["kernel"])
     if dom_key[1] == 2:  # B (m^2), X^T read twice (operand + addend), X' and X'^T written: bf16
         per = [(min(s) ** 2 + 4 * min(s) * max(s)) * 2.0 for s in shapes]
-        roofline["algorithmic_bytes_per_launch"] = sum(per) * (4 if not dom_key[3] else 1) / 5 / dom["n"]
+        roofline["algorithmic_bytes_per_launch"] = sum(per) * (4 if not dom_key[3] else 1) / dom["n"]
     gemm_ms = sum(d["ms"] for d in by_kernel.values())
     f_issued = sum(d["fi"] for d in by_kernel.values())
     hbm = {}

@@ -1,0 +1,150 @@
+"""The benchmark configurations at FULL size on the GPU, checked through size-independent properties and against
+the CPU oracle on sampled matrices (the oracle finishes those in seconds).
+
+config 2: full MuonH step over the depth-16 dense parameter set (112 matrices, 721 M elements)
+config 4: large-matrix NS5 on heavy-tailed gradients with zeroed rows (8192x8192, 4096x14336)
+config 5: full MuonH step for the depth-24 MoE parameter set (6.3 G elements; 3-D expert stacks)
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import muon_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+NS_TOL = 1e-2
+W_TOL = 2e-2
+
+
+def _rel(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return ((a - b).norm() / b.norm()).item()
+
+
+def _oracle_muonh(w, g, m, **kw):
+    x, mm = w.clone(), m.clone()
+    O.lit_gpt_muon_step(x, g, mm, lr=0.02, mu=0.95, wd=0.0, eps=1e-8, nesterov=True, adjust="spectral_norm",
+                        flatten=False, cautious=False, use_muonh=True, **kw)
+    return x, mm
+
+
+def test_config2_full_step(gpu_device):
+    from archscale_amd.optim.muon import Muon
+    layer = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (5632, 2048), (5632, 2048), (2048, 5632)]
+    g = torch.Generator(device=gpu_device).manual_seed(1236)
+    params, grads = [], []
+    for _ in range(16):
+        for s in layer:
+            params.append(torch.nn.Parameter((torch.randn(*s, generator=g, device=gpu_device) * 0.02).to(torch.bfloat16)))
+            grads.append((torch.randn(*s, generator=g, device=gpu_device) * 1e-3).to(torch.bfloat16))
+    for p, gr in zip(params, grads):
+        p.grad = gr
+    opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, use_muonh=True)
+    sample = [1, 6, 4, 59, 111]  # a Wk, a W2 (wide), a W1 (tall), and two more
+    w0 = {i: params[i].detach().cpu().clone() for i in sample}
+    norms0 = torch.stack([p.detach().float().norm() for p in params])
+    # two steps, so that the second one runs with momentum != gradient
+    opt.step()
+    w1 = {i: params[i].detach().cpu().clone() for i in sample}
+    m1 = {i: opt.state[params[i]]["momentum"].detach().cpu().clone() for i in sample}
+    norms1 = torch.stack([p.detach().float().norm() for p in params])
+    opt.step()
+    torch.cuda.synchronize()
+    norms2 = torch.stack([p.detach().float().norm() for p in params])
+    # hypersphere: every matrix keeps its Frobenius norm (bf16 weights: rounding noise only)
+    assert ((norms1 / norms0 - 1).abs().max().item() < 2e-3) and ((norms2 / norms0 - 1).abs().max().item() < 3e-3)
+    for i in sample:
+        x1, mm1 = _oracle_muonh(w0[i], grads[i].cpu(), torch.zeros_like(w0[i]), ns_storage="fp32")
+        assert _rel(w1[i], x1) <= W_TOL
+        assert _rel(w1[i], x1) < 0.3 * _rel(w0[i], x1)        # the step is really there (a no-op sits at ~lr)
+        assert _rel(m1[i], mm1) < 1e-6
+        # second step from the GPU's own state after step 1
+        x2, _ = _oracle_muonh(w1[i], grads[i].cpu(), m1[i], ns_storage="fp32")
+        assert _rel(params[i].detach(), x2) <= W_TOL
+        assert _rel(params[i].detach(), x2) < 0.3 * _rel(w1[i], x2)
+    assert opt.param_groups[0]["step"] == 2
+
+
+def _heavy_tailed(shape, seed):
+    """Student-t(df=3) scaled to std 1e-3, 1 % of the rows zeroed (exercises the norm epsilon and fp32 accumulation)."""
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(*shape, generator=g)
+    chi = torch.randn(3, *shape, generator=g).square().sum(0)
+    t = z / (chi / 3).sqrt() / math.sqrt(3.0) * 1e-3
+    rows = torch.randperm(shape[0], generator=g)[: max(1, shape[0] // 100)]
+    t[rows] = 0
+    return t.to(torch.bfloat16), rows
+
+
+@pytest.mark.parametrize("shape,seed", [((4096, 14336), 1238), ((8192, 8192), 1239)])
+@pytest.mark.parametrize("table", ["quintic", "simple"])
+def test_config4_large_heavy_tailed(gpu_device, shape, seed, table):
+    import archscale_amd.optim.newton_schulz_hip as H
+    G, zero_rows = _heavy_tailed(shape, seed)
+    coeffs = O.coefficient_schedule(table, 5)
+    got = H.newton_schulz(G.to(gpu_device), coeffs, 1e-7, prec="bsplit" if table == "simple" else "bf16")
+    torch.cuda.synchronize()
+    got = got.cpu()
+    assert torch.all(got[zero_rows] == 0)
+    assert torch.isfinite(got.float()).all()
+    if shape == (4096, 14336) or table == "quintic":
+        # full fp32 oracle on the host (seconds for 4096x14336, under a minute for 8192^2)
+        want = O.newton_schulz(G, coeffs, 1e-7, storage="fp32")
+        assert _rel(got, want) <= NS_TOL
+    # squared row norms are the diagonal of O O^T = U p(S)^2 U^T: bounded by the square of the band's upper end,
+    # and their sum is the number of singular values pushed to ~1 (the rank, here the non-zero rows)
+    sq = got.float().square().sum(dim=1)
+    assert sq.max().item() <= 1.25 ** 2
+    rank = shape[0] - len(zero_rows)
+    assert 0.6 * rank <= sq.sum().item() <= 1.25 ** 2 * rank
+
+
+def test_config5_moe_full_step(gpu_device):
+    """24 layers x {Wq, Wo 3072^2; Wk, Wv 768x3072; shared W1, W3 1536x3072, W2 3072x1536; routed experts
+    (64, 768, 3072) and (64, 3072, 384)}: 6.34 G elements in bf16. Reports step time and HBM footprint."""
+    from archscale_amd.optim.muon import Muon
+    free, total = torch.cuda.mem_get_info()
+    if free < 150 << 30:
+        pytest.skip("needs ~110 GiB of free HBM")
+    layer = [(3072, 3072), (768, 3072), (768, 3072), (3072, 3072), (1536, 3072), (1536, 3072), (3072, 1536),
+             (64, 768, 3072), (64, 3072, 384)]
+    g = torch.Generator(device=gpu_device).manual_seed(1240)
+    params, grads = [], []
+    for _ in range(24):
+        for s in layer:
+            params.append(torch.nn.Parameter((torch.randn(*s, generator=g, device=gpu_device) * 0.02).to(torch.bfloat16)))
+            grads.append((torch.randn(*s, generator=g, device=gpu_device) * 1e-3).to(torch.bfloat16))
+    n_elem = sum(p.numel() for p in params)
+    assert n_elem == 24 * (2 * 3072 ** 2 + 2 * 768 * 3072 + 3 * 1536 * 3072 + 64 * 768 * 3072 + 64 * 3072 * 384)
+    for p, gr in zip(params, grads):
+        p.grad = gr
+    opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, use_muonh=True,
+               muonh_per_matrix=True)
+    sample = [(0, None), (6, None), (7, 5), (8, 63), (9 * 23 + 7, 0), (9 * 23 + 8, 31)]
+    w0 = {}
+    for i, e in sample:
+        w0[(i, e)] = (params[i] if e is None else params[i][e]).detach().cpu().clone()
+    n0 = params[7].detach().float().flatten(1).norm(dim=1)
+    torch.cuda.synchronize()
+    opt.step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    opt.step()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1)
+    peak = torch.cuda.max_memory_allocated() / 2 ** 30
+    print(f"config 5: {n_elem / 1e9:.2f} G elements, second step {ms:.1f} ms, peak HBM allocated {peak:.1f} GiB", flush=True)
+    n2 = params[7].detach().float().flatten(1).norm(dim=1)
+    assert (n2 / n0 - 1).abs().max().item() < 3e-3          # every expert keeps its own norm
+    for i, e in sample:
+        gr = (grads[i] if e is None else grads[i][e]).cpu()
+        x1, m1 = _oracle_muonh(w0[(i, e)], gr, torch.zeros_like(gr), ns_storage="fp32")
+        x2, _ = _oracle_muonh(x1, gr, m1, ns_storage="fp32")
+        got = (params[i] if e is None else params[i][e]).detach()
+        # two steps of 2e-2 each: the oracle chain and the GPU chain stay within the single-step bar of each other
+        assert _rel(got, x2) <= W_TOL
+        assert _rel(got, x2) < 0.3 * _rel(w0[(i, e)], x2)
