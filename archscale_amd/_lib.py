@@ -31,6 +31,14 @@ POST_ITEM = np.dtype(
 assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32
 
 
+class NsProblem(ctypes.Structure):
+    """muon_ns_problem of include/archscale_muon.h."""
+    _fields_ = [("in_ptr", ctypes.c_void_p), ("out_ptr", ctypes.c_void_p),
+                ("in_batch_stride", ctypes.c_int64), ("out_batch_stride", ctypes.c_int64),
+                ("in_dtype", ctypes.c_int32), ("in_ld", ctypes.c_int32), ("out_ld", ctypes.c_int32),
+                ("batch", ctypes.c_int32), ("rows", ctypes.c_int32), ("cols", ctypes.c_int32)]
+
+
 class MuonLibraryError(RuntimeError):
     """The HIP library is missing, has the wrong ABI, or a call into it failed."""
 
@@ -46,6 +54,11 @@ _SIGNATURES = {
         ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_ns_grouped_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(NsProblem), ctypes.c_int, ctypes.c_int]),
+    "muon_ns_grouped": (ctypes.c_int, [
+        ctypes.POINTER(NsProblem), ctypes.c_int,
         ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_ns_flops": (None, [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 3),

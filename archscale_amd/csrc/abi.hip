@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <mutex>
 #include <vector>
 
@@ -75,9 +76,9 @@ std::mutex g_prof_mutex;
 std::vector<ProfRec> g_prof;
 bool g_prof_on = false;
 
-hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GemmParams& g, hipStream_t stream,
+hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GroupedGemmParams& g, hipStream_t stream,
                       double flops_algorithmic, double flops_issued) {
-  if (!g_prof_on) return launch_ns_gemm(tile, mode, split, final_, g, stream);
+  if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   ProfRec r;
   r.key = tile * 100 + mode * 10 + (split ? 2 : 0) + (final_ ? 1 : 0);
@@ -87,7 +88,7 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GemmPar
   if ((e = hipEventCreate(&r.start)) != hipSuccess) return e;
   if ((e = hipEventCreate(&r.stop)) != hipSuccess) return e;
   if ((e = hipEventRecord(r.start, stream)) != hipSuccess) return e;
-  e = launch_ns_gemm(tile, mode, split, final_, g, stream);
+  e = launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
   hipError_t e2 = hipEventRecord(r.stop, stream);
   g_prof.push_back(r);
   return e != hipSuccess ? e : e2;
@@ -127,86 +128,201 @@ void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode, doub
   }
 }
 
-int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld, void* out_dev,
-                    int64_t out_batch_stride, int out_ld, int batch, int rows, int cols, const float* abc_host,
-                    int iters, float eps, int eps_mode, int prec_mode, int flags, void* ws_dev, size_t ws_bytes,
-                    void* stream_) {
+// plan + carved workspace pointers of one problem of a grouped call
+namespace {
+struct NsProblem {
+  muon_ns_problem q;
+  NsPlan pl;
+  __bf16 *X[2], *Xt[2], *A, *Bh, *Bl;
+  float *partial, *scale;
+  bool tall;
+};
+
+int check_problem(const muon_ns_problem& q) {
+  if (!q.in || !q.out) return MUON_E_ARG;
+  if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return MUON_E_ARG;
+  if (q.in_ld < q.cols || q.out_ld < q.cols) return MUON_E_ARG;
+  if (q.in_dtype != MUON_DTYPE_BF16 && q.in_dtype != MUON_DTYPE_F32) return MUON_E_ARG;
+  return 0;
+}
+}  // namespace
+
+size_t muon_ns_grouped_workspace_bytes(const muon_ns_problem* problems_host, int n_problems, int prec_mode) {
+  if (!problems_host || n_problems <= 0) return 0;
+  size_t total = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    const muon_ns_problem& q = problems_host[i];
+    if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return 0;
+    total += make_plan(q.batch, q.rows, q.cols, prec_mode).total;
+  }
+  return total;
+}
+
+int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const float* abc_host, int iters, float eps,
+                    int eps_mode, int prec_mode, int flags, void* ws_dev, size_t ws_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  if (!in_dev || !out_dev || !abc_host || !ws_dev) return MUON_E_ARG;
-  if (batch <= 0 || rows <= 0 || cols <= 0 || iters <= 0) return MUON_E_ARG;
-  if (in_ld < cols || out_ld < cols) return MUON_E_ARG;
-  if (in_dtype != MUON_DTYPE_BF16 && in_dtype != MUON_DTYPE_F32) return MUON_E_ARG;
+  if (!problems_host || n_problems <= 0 || !abc_host || !ws_dev || iters <= 0) return MUON_E_ARG;
   if (eps_mode != MUON_EPS_ADD && eps_mode != MUON_EPS_CLAMP) return MUON_E_ARG;
   if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT) return MUON_E_ARG;
-  const NsPlan pl = make_plan(batch, rows, cols, prec_mode);
-  if (ws_bytes < pl.total || ((uintptr_t)ws_dev & 255)) return MUON_E_WORKSPACE;
-  // byte offsets inside one matrix are 32-bit in the GEMM loader
-  if ((double)pl.Mp * pl.Np * 2.0 >= 4294967296.0) return MUON_E_UNSUPPORTED;
+  if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
+  const bool split = prec_mode == MUON_PREC_BF16_BSPLIT;
+  const int cast_first = (flags & MUON_NS_CAST_INPUT_FIRST) ? 1 : 0;
 
-  char* ws = (char*)ws_dev;
-  __bf16* X[2] = {(__bf16*)(ws + pl.off_x[0]), (__bf16*)(ws + pl.off_x[1])};
-  __bf16* Xt[2] = {(__bf16*)(ws + pl.off_xt[0]), (__bf16*)(ws + pl.off_xt[1])};
-  __bf16* A = (__bf16*)(ws + pl.off_a);
-  __bf16* Bh = (__bf16*)(ws + pl.off_bh);
-  __bf16* Bl = prec_mode == MUON_PREC_BF16_BSPLIT ? (__bf16*)(ws + pl.off_bl) : nullptr;
-  float* partial = (float*)(ws + pl.off_partial);
-  float* scale = (float*)(ws + pl.off_scale);
-  const bool split = Bl != nullptr;
-  const bool tall = rows > cols;
-  const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
+  std::vector<NsProblem> pr(n_problems);
+  size_t off = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    NsProblem& P = pr[i];
+    P.q = problems_host[i];
+    const int st = check_problem(P.q);
+    if (st) return st;
+    P.pl = make_plan(P.q.batch, P.q.rows, P.q.cols, prec_mode);
+    // byte offsets inside one matrix are 32-bit in the GEMM loader
+    if ((double)P.pl.Mp * P.pl.Np * 2.0 >= 4294967296.0) return MUON_E_UNSUPPORTED;
+    if (off + P.pl.total > ws_bytes) return MUON_E_WORKSPACE;
+    char* ws = (char*)ws_dev + off;
+    off += P.pl.total;
+    P.X[0] = (__bf16*)(ws + P.pl.off_x[0]); P.X[1] = (__bf16*)(ws + P.pl.off_x[1]);
+    P.Xt[0] = (__bf16*)(ws + P.pl.off_xt[0]); P.Xt[1] = (__bf16*)(ws + P.pl.off_xt[1]);
+    P.A = (__bf16*)(ws + P.pl.off_a);
+    P.Bh = (__bf16*)(ws + P.pl.off_bh);
+    P.Bl = split ? (__bf16*)(ws + P.pl.off_bl) : nullptr;
+    P.partial = (float*)(ws + P.pl.off_partial);
+    P.scale = (float*)(ws + P.pl.off_scale);
+    P.tall = P.q.rows > P.q.cols;
+  }
+  // launch order inside a grouped kernel: problems with the longest tiles first, so the tail of the
+  // grid is made of short tiles
+  std::vector<int> order(n_problems);
+  for (int i = 0; i < n_problems; ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    return (long)pr[a].pl.Mp * pr[a].pl.Np > (long)pr[b].pl.Mp * pr[b].pl.Np;
+  });
 
   // normalise; the input's own orientation goes to X (wide) or X^T (tall), its transpose to the other
-  const int cast_first = (flags & MUON_NS_CAST_INPUT_FIRST) ? 1 : 0;
-  hipError_t e = launch_norm_scale(in_dev, in_dtype, cast_first, in_batch_stride, in_ld, batch, rows, cols, eps,
-                                   eps_mode, partial, scale, stream);
-  if (e != hipSuccess) return (int)e;
-  if (!tall)
-    e = launch_layout(in_dev, in_dtype, cast_first, in_batch_stride, in_ld, batch, rows, cols, scale, X[0], xs,
-                      pl.Np, pl.Mp, pl.Np, Xt[0], xs, pl.Mp, stream);
-  else
-    e = launch_layout(in_dev, in_dtype, cast_first, in_batch_stride, in_ld, batch, rows, cols, scale, Xt[0], xs,
-                      pl.Mp, pl.Np, pl.Mp, X[0], xs, pl.Np, stream);
-  if (e != hipSuccess) return (int)e;
+  hipError_t e;
+  for (int i = 0; i < n_problems; ++i) {
+    const NsProblem& P = pr[i];
+    const NsPlan& pl = P.pl;
+    const long xs = (long)pl.Mp * pl.Np;
+    e = launch_norm_scale(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
+                          P.q.cols, eps, eps_mode, P.partial, P.scale, stream);
+    if (e != hipSuccess) return (int)e;
+    if (!P.tall)
+      e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
+                        P.q.cols, P.scale, P.X[0], xs, pl.Np, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
+    else
+      e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
+                        P.q.cols, P.scale, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, P.X[0], xs, pl.Np, stream);
+    if (e != hipSuccess) return (int)e;
+  }
 
-  const int tm = pl.Mp / pl.tile, tn = pl.Np / pl.tile;
+  // one product of the iteration for every problem: problems that share a tile configuration go into one
+  // launch (at most MAX_GROUPS per launch)
+  auto run_mode = [&](int mode, bool last, auto&& fill) -> hipError_t {
+    for (int tile : {256, 128}) {
+      GroupedGemmParams gp = {};
+      double fa = 0.0, fi = 0.0;
+      auto flush = [&]() -> hipError_t {
+        if (gp.n_groups == 0) return hipSuccess;
+        hipError_t err = timed_gemm(tile, mode, split && mode != MODE_SYRK, last && mode == MODE_BX, gp, stream, fa, fi);
+        gp = GroupedGemmParams{};
+        fa = fi = 0.0;
+        return err;
+      };
+      for (int oi = 0; oi < n_problems; ++oi) {
+        const NsProblem& P = pr[order[oi]];
+        if (P.pl.tile != tile) continue;
+        GemmParams g = {};
+        double a_fl = 0.0, i_fl = 0.0;
+        fill(P, g, a_fl, i_fl);
+        const long tiles = ns_gemm_tiles(mode, g);
+        if (tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L || gp.n_groups == MAX_GROUPS) {
+          hipError_t err = flush();
+          if (err != hipSuccess) return err;
+        }
+        if (tiles > 0x7ffffff0L) return hipErrorInvalidValue;
+        gp.g[gp.n_groups] = g;
+        gp.tile_start[gp.n_groups + 1] = gp.tile_start[gp.n_groups] + (int)tiles;
+        ++gp.n_groups;
+        fa += a_fl;
+        fi += i_fl;
+      }
+      hipError_t err = flush();
+      if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
+  };
+
   int cur = 0;
   for (int it = 0; it < iters; ++it) {
     const float a = abc_host[3 * it], b = abc_host[3 * it + 1], c = abc_host[3 * it + 2];
     const bool last = it == iters - 1;
-    GemmParams g = {};
-    g.batch = batch;
     // A = X X^T
-    g.P = X[cur]; g.Q = X[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
-    g.tilesM = g.tilesN = tm;
-    g.C = A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
-    const double bm = (double)batch, dm = pl.m, dn = pl.n, tl = pl.tile;
-    const double st = (double)sym_tiles(tm);
-    if ((e = timed_gemm(pl.tile, MODE_SYRK, false, false, g, stream, bm * dm * dm * dn,
-                        bm * 2.0 * tl * tl * st * pl.Np)) != hipSuccess) return (int)e;
+    e = run_mode(MODE_SYRK, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      const NsPlan& pl = P.pl;
+      const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
+      g.batch = P.q.batch;
+      g.P = P.X[cur]; g.Q = P.X[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
+      g.tilesM = g.tilesN = pl.Mp / pl.tile;
+      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
+      const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
+      fa = bm * dm * dm * dn;
+      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
+    });
+    if (e != hipSuccess) return (int)e;
     // B = c A A + b A
-    g.P = A; g.Q = A; g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
-    g.E = A; g.strideE = as; g.lde = pl.Mp;
-    g.C = Bh; g.C2 = Bl; g.alpha = c; g.beta = b;
-    if ((e = timed_gemm(pl.tile, MODE_SYRK2, split, false, g, stream, bm * dm * dm * dm,
-                        bm * 2.0 * tl * tl * st * pl.Mp)) != hipSuccess) return (int)e;
+    e = run_mode(MODE_SYRK2, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      const NsPlan& pl = P.pl;
+      const long as = (long)pl.Mp * pl.Mp;
+      g.batch = P.q.batch;
+      g.P = P.A; g.Q = P.A; g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
+      g.tilesM = g.tilesN = pl.Mp / pl.tile;
+      g.E = P.A; g.strideE = as; g.lde = pl.Mp;
+      g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp; g.alpha = c; g.beta = b;
+      const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
+      fa = bm * dm * dm * dm;
+      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
+    });
+    if (e != hipSuccess) return (int)e;
     // X' = a X + B X
-    g.P = Bh; g.P2 = Bl; g.Q = Xt[cur]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp; g.K = pl.Mp;
-    g.tilesM = tm; g.tilesN = tn;
-    g.E = Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
-    g.alpha = a; g.beta = 0.f; g.C2 = nullptr;
-    if (!last) {
-      g.C = X[cur ^ 1]; g.strideC = xs; g.ldc = pl.Np;
-      g.Ct = Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;
-    } else {
-      g.m_valid = pl.m; g.n_valid = pl.n;
-      if (!tall) { g.C = (__bf16*)out_dev; g.strideC = out_batch_stride; g.ldc = out_ld; g.Ct = nullptr; }
-      else { g.C = nullptr; g.Ct = (__bf16*)out_dev; g.strideCt = out_batch_stride; g.ldct = out_ld; }
-    }
-    if ((e = timed_gemm(pl.tile, MODE_BX, split, last, g, stream, bm * 2.0 * dm * dm * dn,
-                        bm * 2.0 * tl * tl * tm * tn * pl.Mp * (split ? 2.0 : 1.0))) != hipSuccess) return (int)e;
+    e = run_mode(MODE_BX, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      const NsPlan& pl = P.pl;
+      const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
+      g.batch = P.q.batch;
+      g.P = P.Bh; g.P2 = P.Bl; g.Q = P.Xt[cur]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp;
+      g.K = pl.Mp;
+      g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
+      g.E = P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
+      g.alpha = a; g.beta = 0.f;
+      if (!last) {
+        g.C = P.X[cur ^ 1]; g.strideC = xs; g.ldc = pl.Np;
+        g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;
+      } else {
+        g.m_valid = pl.m; g.n_valid = pl.n;
+        if (!P.tall) { g.C = (__bf16*)P.q.out; g.strideC = P.q.out_batch_stride; g.ldc = P.q.out_ld; }
+        else { g.Ct = (__bf16*)P.q.out; g.strideCt = P.q.out_batch_stride; g.ldct = P.q.out_ld; }
+      }
+      const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
+      fa = bm * 2.0 * dm * dm * dn;
+      fi = bm * 2.0 * tl * tl * (double)(pl.Mp / pl.tile) * (pl.Np / pl.tile) * pl.Mp * (split ? 2.0 : 1.0);
+    });
+    if (e != hipSuccess) return (int)e;
     cur ^= 1;
   }
   return 0;
+}
+
+int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld, void* out_dev,
+                    int64_t out_batch_stride, int out_ld, int batch, int rows, int cols, const float* abc_host,
+                    int iters, float eps, int eps_mode, int prec_mode, int flags, void* ws_dev, size_t ws_bytes,
+                    void* stream) {
+  muon_ns_problem q;
+  q.in = in_dev; q.out = out_dev;
+  q.in_batch_stride = in_batch_stride; q.out_batch_stride = out_batch_stride;
+  q.in_dtype = in_dtype; q.in_ld = in_ld; q.out_ld = out_ld;
+  q.batch = batch; q.rows = rows; q.cols = cols;
+  if (!ws_dev) return MUON_E_ARG;
+  return muon_ns_grouped(&q, 1, abc_host, iters, eps, eps_mode, prec_mode, flags, ws_dev, ws_bytes, stream);
 }
 
 size_t muon_syrk_workspace_bytes(int batch, int n, int k) {

@@ -31,7 +31,22 @@ struct GemmParams {
   int m_valid, n_valid;  // true extents for the bounds-checked final store
 };
 
+// Several independent problems of one kind (same tile configuration, mode, split and final flags) in ONE
+// launch: block b works on problem g with tile_start[g] <= b < tile_start[g+1].  Passed by value as a
+// kernel argument (about 1.3 KiB).
+constexpr int MAX_GROUPS = 8;
+struct GroupedGemmParams {
+  int n_groups;
+  int tile_start[MAX_GROUPS + 1];
+  GemmParams g[MAX_GROUPS];
+};
+
+// number of block tiles of one problem
+long ns_gemm_tiles(int mode, const GemmParams& p);
+
 // tile: 256 (256x256 block tile, 8 waves) or 128 (128x128, 4 waves)
+hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
+                                  hipStream_t stream);
 hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream);
 
 }  // namespace archscale

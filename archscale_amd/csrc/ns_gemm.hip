@@ -55,7 +55,7 @@ __device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * ROW_BYTE
 
 template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
-ns_gemm_kernel(const GemmParams p) {
+ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int WAVES_N = BN / WN;
   constexpr int FM = WM / 32, FN = WN / 32;
@@ -73,14 +73,20 @@ ns_gemm_kernel(const GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
 
-  // ---- block -> (matrix, tile) : consecutive logical tiles share an XCD (and its L2)
-  const int nblk = gridDim.x;  // multiple of 8
-  const int per_xcd = nblk >> 3;
-  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  // ---- block -> (problem, matrix, tile).  Workgroups are dealt round-robin to the 8 XCDs; runs of 32
+  // consecutive logical tiles (neighbouring tiles of one matrix: shared operand panels) are kept on ONE
+  // XCD, i.e. in one L2, and successive runs go to successive XCDs so that long and short tiles of a
+  // grouped launch spread evenly over the chip.  The grid is a multiple of 8*32.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int logical = (((slot >> 5) << 3) + xcd) * 32 + (slot & 31);
+  if (logical >= gp.tile_start[gp.n_groups]) return;
+  int grp = 0;
+  while (grp + 1 < gp.n_groups && logical >= gp.tile_start[grp + 1]) ++grp;
+  const GemmParams p = gp.g[grp];
+  const int local = logical - gp.tile_start[grp];
   const int tiles_per_mat = SYM ? (p.tilesM * (p.tilesM + 1)) / 2 : p.tilesM * p.tilesN;
-  if (logical >= p.batch * tiles_per_mat) return;
-  const int b = logical / tiles_per_mat;
-  int t = logical - b * tiles_per_mat;
+  const int b = local / tiles_per_mat;
+  int t = local - b * tiles_per_mat;
   int ti, tj;
   if (SYM) {
     ti = 0;
@@ -358,8 +364,13 @@ ns_gemm_kernel(const GemmParams p) {
 // ---------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------
+long ns_gemm_tiles(int mode, const GemmParams& p) {
+  const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2);
+  return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
+}
+
 template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL>
-static hipError_t launch_one(const GemmParams& p, hipStream_t stream) {
+static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
   auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL>;
@@ -369,17 +380,15 @@ static hipError_t launch_one(const GemmParams& p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const bool sym = (MODE == MODE_SYRK || MODE == MODE_SYRK2);
-  const long tiles = (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
+  const long tiles = gp.tile_start[gp.n_groups];
   if (tiles <= 0) return hipSuccess;
-  const long grid = (tiles + 7) / 8 * 8;
-  if (grid > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), SMEM, stream, p);
+  const long grid = (tiles + 255) / 256 * 256;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), SMEM, stream, gp);
   return hipGetLastError();
 }
 
 template <int BM, int BN, int WM, int WN>
-static hipError_t launch_cfg(int mode, bool split, bool final_, const GemmParams& p, hipStream_t s) {
+static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGemmParams& p, hipStream_t s) {
   switch (mode) {
     case MODE_SYRK:
       return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false>(p, s);
@@ -396,11 +405,24 @@ static hipError_t launch_cfg(int mode, bool split, bool final_, const GemmParams
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream) {
-  if (p.K % BK != 0 || p.K <= 0) return hipErrorInvalidValue;
-  if (tile == 256) return launch_cfg<256, 256, 128, 64>(mode, split, final_, p, stream);
-  if (tile == 128) return launch_cfg<128, 128, 64, 64>(mode, split, final_, p, stream);
+hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
+                                  hipStream_t stream) {
+  if (gp.n_groups < 1 || gp.n_groups > MAX_GROUPS) return hipErrorInvalidValue;
+  for (int i = 0; i < gp.n_groups; ++i)
+    if (gp.g[i].K % BK != 0 || gp.g[i].K <= 0 || gp.tile_start[i + 1] < gp.tile_start[i]) return hipErrorInvalidValue;
+  if (tile == 256) return launch_cfg<256, 256, 128, 64>(mode, split, final_, gp, stream);
+  if (tile == 128) return launch_cfg<128, 128, 64, 64>(mode, split, final_, gp, stream);
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream) {
+  GroupedGemmParams gp = {};
+  gp.n_groups = 1;
+  gp.g[0] = p;
+  const long tiles = ns_gemm_tiles(mode, p);
+  if (tiles > 0x7ffffff0L) return hipErrorInvalidValue;
+  gp.tile_start[1] = (int)tiles;
+  return launch_ns_gemm_grouped(tile, mode, split, final_, gp, stream);
 }
 
 }  // namespace archscale

@@ -376,9 +376,8 @@ class Muon(Optimizer):
                                            1.0 if nesterov else 0.0, 0.0, stream), "muon_momentum")
             # U <- NS(U), one batched call per shape class                    (muon.py:821-838)
             if self._newton_schulz_func is None:
-                for cls in plan.classes.values():
-                    with self._timed(f"newton_schulz[{cls.n_mats}x{cls.rows}x{cls.cols}]"):
-                        self._orthogonalize_class(cls, eps)
+                with self._timed("newton_schulz"):
+                    self._orthogonalize_classes(list(plan.classes.values()), eps)
             else:
                 self._orthogonalize_with_hook(plan, eps)
             # weight update                                                   (muon.py:598-650)
@@ -393,14 +392,33 @@ class Muon(Optimizer):
                                                    len(plan.post_rows), plan.post_chunks, lr, lr * wd, int(cautious),
                                                    stream), "muon_update_plain")
 
-    def _orthogonalize_class(self, cls: _ShapeClass, eps: float) -> None:
+    def _orthogonalize_classes(self, classes: List[_ShapeClass], eps: float) -> None:
+        """U <- NS(U) for every shape class in ONE grouped call (each product of the iteration is one launch over
+        all classes); classes are sliced / the call is split only when the workspace would exceed the limit."""
         L = _lib.lib()
         pm = _lib.PREC_BF16_BSPLIT if self._ns_precision == "bsplit" else _lib.PREC_BF16
-        per = max(1, L.muon_ns_workspace_bytes(1, cls.rows, cls.cols, pm))
-        step = max(1, min(cls.n_mats, self._ns_workspace_limit // per))
-        for lo in range(0, cls.n_mats, step):
-            part = cls.U[lo:lo + step]
-            ns.newton_schulz(part, self._ns_coefficients, eps, prec=self._ns_precision, out=part)
+        parts: List[Tensor] = []
+        used = 0
+
+        def run():
+            nonlocal parts, used
+            if parts:
+                ns.newton_schulz_grouped(parts, self._ns_coefficients, eps, prec=self._ns_precision, outs=parts)
+            parts, used = [], 0
+
+        for cls in classes:
+            per = max(1, L.muon_ns_workspace_bytes(1, cls.rows, cls.cols, pm))
+            lo = 0
+            while lo < cls.n_mats:
+                room = (self._ns_workspace_limit - used) // per
+                if room < 1 and parts:
+                    run()
+                    continue
+                take = max(1, min(cls.n_mats - lo, room))
+                parts.append(cls.U[lo:lo + take])
+                used += take * per
+                lo += take
+        run()
 
     def _orthogonalize_with_hook(self, plan: _GroupPlan, eps: float) -> None:
         # user hook, one tensor at a time with the reference's flatten policy (muon.py:821-838);

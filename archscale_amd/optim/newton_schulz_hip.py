@@ -104,6 +104,52 @@ def newton_schulz(
     return out
 
 
+def newton_schulz_grouped(
+    inputs: Sequence[Tensor],
+    coeffs: Coeffs = QUINTIC_SCHEDULE,
+    epsilon: Union[float, Tensor] = 1e-7,
+    *,
+    eps_mode: str = "add",
+    prec: str = "bf16",
+    cast_input_first: bool = True,
+    outs: Optional[Sequence[Tensor]] = None,
+) -> Sequence[Tensor]:
+    """Orthogonalise several batches of DIFFERENT shapes in one call: every product of the iteration is a
+    single kernel launch over the tiles of all batches (15 GEMM launches in total for five iterations).
+    ``inputs[i]`` is ``[..., rows_i, cols_i]`` (bf16 or fp32); ``outs[i]`` (bf16, contiguous, may be the input)
+    receives the result.  All tensors must live on one device."""
+    if not inputs:
+        return []
+    device = inputs[0].device
+    views = []
+    for G in inputs:
+        _lib.require_cuda(G, "Newton-Schulz input")
+        if G.device != device:
+            raise ValueError("all inputs of a grouped call must live on one device")
+        if G.dtype not in (torch.bfloat16, torch.float32):
+            G = G.to(torch.float32)
+        views.append((G.shape, *_as_batch(G)))
+    if outs is None:
+        outs = [torch.empty(shape, dtype=torch.bfloat16, device=device) for shape, *_ in views]
+    probs = (_lib.NsProblem * len(views))()
+    for q, (shape, Gv, batch, rows, cols, bstride, ld), out in zip(probs, views, outs):
+        if out.shape != shape or out.dtype != torch.bfloat16 or not out.is_contiguous() or out.device != device:
+            raise ValueError("every out must be a contiguous bfloat16 tensor shaped like its input, on the same device")
+        q.in_ptr, q.out_ptr = Gv.data_ptr(), out.data_ptr()
+        q.in_batch_stride, q.out_batch_stride = bstride, rows * cols
+        q.in_dtype, q.in_ld, q.out_ld = _lib.dtype_code(Gv.dtype), ld, cols
+        q.batch, q.rows, q.cols = batch, rows, cols
+    L = _lib.lib()
+    pm = _PREC[prec]
+    ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(probs, len(views), pm))
+    flags = _lib.NS_CAST_INPUT_FIRST if cast_input_first else 0
+    with torch.cuda.device(device):
+        st = L.muon_ns_grouped(probs, len(views), _lib.abc_array(coeffs), len(coeffs), _as_float(epsilon),
+                               _EPS[eps_mode], pm, flags, ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(device))
+    _lib.check(st, "muon_ns_grouped")
+    return list(outs)
+
+
 def zeropower_via_newtonschulz5(G: Tensor, epsilon: Union[float, Tensor] = 1e-7) -> Tensor:
     """Drop-in for lit_gpt/optim/muon.py:869-897 (five iterations, production coefficient schedule)."""
     return newton_schulz(G, QUINTIC_SCHEDULE, epsilon)

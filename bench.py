@@ -209,7 +209,7 @@ def main():
             gbs = n_elem * bytes_per_elem[name] / ms / 1e6
             hbm[name] = {"ms": round(ms, 3), "GB/s": round(gbs, 0), "frac": round(gbs / HBM_PEAK_GBS, 3),
                          "bytes_per_elem": bytes_per_elem[name]}
-    ns_ms = sum(ms for n, ms in phases.items() if n.startswith("newton_schulz"))
+    ns_ms = sum(ms for n, ms in phases.items() if n.startswith("newton_schulz"))  # norms, layout and the 15 grouped GEMMs
 
     out = {
         "metric": "Muon NS5 TFLOP/s (% bf16 MFMA peak) + MuonH step ms, d16 param set, 1 GPU",

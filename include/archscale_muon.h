@@ -72,6 +72,24 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
                     const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
                     void* ws_dev, size_t ws_bytes, void* stream);
 
+/* The same for several independent batches of different shapes at once (all shape classes of an optimizer
+ * step): each product of the iteration is ONE kernel launch over the tiles of every problem, so there are
+ * 15 GEMM launches per call whatever the number of shapes, and the tail of one shape's grid is filled by the
+ * next.  Replaces the per-parameter task loop of lit_gpt/optim/muon.py:211-333 around the calls above.
+ * problems_host is a HOST array; the workspace is muon_ns_grouped_workspace_bytes(...) bytes. */
+typedef struct muon_ns_problem {
+  const void* in; /* device, [batch] rows x cols, dtype in_dtype */
+  void* out;      /* device, bf16 */
+  int64_t in_batch_stride, out_batch_stride; /* elements */
+  int32_t in_dtype, in_ld, out_ld, batch, rows, cols;
+} muon_ns_problem;
+
+size_t muon_ns_grouped_workspace_bytes(const muon_ns_problem* problems_host, int n_problems, int prec_mode);
+
+int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems,
+                    const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
+                    void* ws_dev, size_t ws_bytes, void* stream);
+
 /* Algorithmic work of one call, for roofline accounting: dense-count FLOPs (what a GEMM library executes),
  * symmetric-count FLOPs (upper-triangle SYRK minimum) and FLOPs this library issues (tiles incl. padding,
  * full diagonal tiles and the second pass of the B split). */

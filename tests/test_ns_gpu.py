@@ -127,6 +127,26 @@ def test_in_place_out(ns, gpu_device):
     assert torch.equal(buf, ref)
 
 
+def test_grouped_equals_separate(ns, gpu_device):
+    """All shape classes in one grouped call (one launch per product over every class) give bit-identical
+    results to one call per class; mixes both tile configurations, tall and wide, 2-D and 3-D, fp32 input."""
+    ins = [_randn((3, 256, 768), 31), _randn((640, 128), 32), _randn((2, 128, 1024), 33), _randn((1024, 1024), 34),
+           torch.randn(100, 200, generator=torch.Generator().manual_seed(35))]
+    ins = [t.to(gpu_device) for t in ins]
+    for prec, coeffs in (("bf16", O.QUINTIC), ("bsplit", O.coefficient_schedule("simple", 5))):
+        sep = [ns.newton_schulz(t, coeffs, 1e-7, prec=prec) for t in ins]
+        grp = ns.newton_schulz_grouped(ins, coeffs, 1e-7, prec=prec)
+        for a, b in zip(sep, grp):
+            assert torch.equal(a, b)
+    # in place, and more problems than fit one launch (9 > 8)
+    many = [_randn((128, 128 * (i + 1)), 40 + i).to(gpu_device) for i in range(9)]
+    want = [ns.newton_schulz(t) for t in many]
+    ns.newton_schulz_grouped(many, outs=many)
+    for a, b in zip(want, many):
+        assert torch.equal(a, b)
+    assert ns.newton_schulz_grouped([]) == []
+
+
 def test_syrk_products(ns, gpu_device):
     X = _randn((2, 192, 320), 21, 0.05).to(gpu_device)
     A = ns.ns_line_1(X)
