@@ -27,6 +27,7 @@ namespace archscale {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -248,6 +249,158 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   auto d_swz = [&](int sr, int ch) { return d_off(sr, ch * 16); };
 
   __syncthreads();  // every wave is done reading the operand stages
+
+  if (!diag) {
+    // ---- wave-local epilogue (every tile except the diagonal tiles of a symmetric product).
+    // Each wave stages its own WM x WN sub-tile in its own LDS region as the transposed image
+    // W[c][r] (c = column in the sub-tile, r = row), so nothing below needs a block barrier:
+    //   addend in:   16-byte direct copies of E[col][row..] rows into W, read back 8 bytes per lane
+    //   W <- values: 8-byte LDS writes (a lane owns 4 consecutive r of one c)
+    //   transposed / mirrored image out: 16-byte reads of W rows -> 16-byte stores, 256 B contiguous per row
+    //   row-major image out: LDS transpose reads (ds_read_b64_tr_b16: a lane receives 4 consecutive c of one
+    //     r; two of them make 16 bytes) -> 16-byte stores, 64 B contiguous per row
+    constexpr int WROW = WM * 2;                  // bytes per W row
+    constexpr int RCH = WM / 8;                   // 16-byte chunks per W row
+    constexpr int WBYTES = WN * WROW;
+    constexpr int WSLABS = WBYTES / 1024;         // 64-chunk slabs of one region
+    static_assert(NW * WBYTES <= 2 * STAGE, "wave regions must fit in the operand stages");
+    char* W = smem + wave * WBYTES;
+    // chunk swizzle: 4 consecutive rows of W land in 4 different pairs of 16-byte bank groups
+    auto sw = [](int c) { return (((c & 7) << 1) | ((c >> 3) & 1)) & (RCH - 1); };
+    auto w_off = [&](int c, int r) { return c * WROW + ((((r >> 3) ^ sw(c)) & (RCH - 1)) << 4) + ((r & 7) << 1); };
+    const int wrow0 = R0 + wr0, wcol0 = C0 + wc0;  // global origin of this wave's sub-tile
+
+    if (MODE != MODE_SYRK) {
+      const char* Eb = (const char*)(p.E + (size_t)b * p.strideE + (size_t)wcol0 * p.lde + wrow0);
+#pragma unroll
+      for (int t = 0; t < WSLABS; ++t) {
+        const int q = t * 64 + lane;
+        const int c = q / RCH, ch = (q % RCH) ^ sw(c);
+        __builtin_amdgcn_global_load_lds((gptr_t)(Eb + ((size_t)c * p.lde + ch * 8) * 2), (lptr_t)(W + t * 1024), 16, 0, 0);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int c = j * 32 + l32;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int r = i * 32 + 8 * g + 4 * hi;
+          if (MODE == MODE_SYRK) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
+          } else {
+            const uint2 e = *(const uint2*)(W + w_off(c, r));
+            const float e0 = bf16_to_f32(e.x & 0xffff), e1 = bf16_to_f32(e.x >> 16);
+            const float e2 = bf16_to_f32(e.y & 0xffff), e3 = bf16_to_f32(e.y >> 16);
+            if (MODE == MODE_SYRK2) {
+              acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
+              acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
+              acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
+              acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
+            } else {
+              acc[i][j][4 * g + 0] += alpha * e0;
+              acc[i][j][4 * g + 1] += alpha * e1;
+              acc[i][j][4 * g + 2] += alpha * e2;
+              acc[i][j][4 * g + 3] += alpha * e3;
+            }
+          }
+        }
+      }
+
+    auto store_wave = [&](__bf16* Cdst) {
+      // W[c][r] <- bf16(acc)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            *(uint2*)(W + w_off(j * 32 + l32, i * 32 + 8 * g + 4 * hi)) =
+                pack4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+      // transposed / mirrored image: rows of W
+      __bf16* Tdst = SYM ? Cdst : p.Ct;
+      if (Tdst) {
+        const long tbs = SYM ? p.strideC : p.strideCt;
+        const int tld = SYM ? p.ldc : p.ldct;
+        __bf16* base = Tdst + (size_t)b * tbs;
+        const bool vec_ok = !FINAL || ((tld & 7) == 0 && (tbs & 7) == 0 && (((uintptr_t)Tdst) & 15) == 0);
+#pragma unroll
+        for (int t = 0; t < WSLABS; ++t) {
+          const int q = t * 64 + lane;
+          const int c = q / RCH, ch = q % RCH;
+          const uint4 val = *(const uint4*)(W + c * WROW + (((ch ^ sw(c)) & (RCH - 1)) << 4));
+          const int orow = wcol0 + c, ocol = wrow0 + ch * 8;   // row of the transposed image = column of the tile
+          if (!FINAL) {
+            *(uint4*)(base + (size_t)orow * tld + ocol) = val;
+          } else if (orow < p.n_valid) {
+            if (vec_ok && ocol + 7 < p.m_valid) {
+              *(uint4*)(base + (size_t)orow * tld + ocol) = val;
+            } else {
+              const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+              for (int k = 0; k < 8; ++k)
+                if (ocol + k < p.m_valid) ((uint16_t*)base)[(size_t)orow * tld + ocol + k] = (uint16_t)(w[k >> 1] >> ((k & 1) * 16));
+            }
+          }
+        }
+      }
+      // row-major image: transpose reads.  In a 16-lane group, source lane s points at W[c0 + s/4][r0 + 4*(s%4) ..+3];
+      // lane L of the group then holds W[c0 .. c0+3][r0 + L].
+      if (SYM || p.C) {
+        __bf16* base = Cdst + (size_t)b * p.strideC;
+        const bool vec_ok = !FINAL || ((p.ldc & 7) == 0 && (p.strideC & 7) == 0 && (((uintptr_t)Cdst) & 15) == 0);
+        const int grp = lane >> 4, s = lane & 15;
+#pragma unroll
+        for (int rb = 0; rb < WM / 16; ++rb)
+#pragma unroll
+          for (int cb = 0; cb < WN / 32; ++cb) {
+            const int c0 = cb * 32 + grp * 8;
+            const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(W + w_off(c0 + (s >> 2), rb * 16 + 4 * (s & 3))));
+            const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(W + w_off(c0 + 4 + (s >> 2), rb * 16 + 4 * (s & 3))));
+            uint4 val;
+            val.x = (uint32_t)(uint16_t)lo4[0] | ((uint32_t)(uint16_t)lo4[1] << 16);
+            val.y = (uint32_t)(uint16_t)lo4[2] | ((uint32_t)(uint16_t)lo4[3] << 16);
+            val.z = (uint32_t)(uint16_t)hi4[0] | ((uint32_t)(uint16_t)hi4[1] << 16);
+            val.w = (uint32_t)(uint16_t)hi4[2] | ((uint32_t)(uint16_t)hi4[3] << 16);
+            const int orow = wrow0 + rb * 16 + s, ocol = wcol0 + c0;
+            if (!FINAL) {
+              *(uint4*)(base + (size_t)orow * p.ldc + ocol) = val;
+            } else if (orow < p.m_valid) {
+              if (vec_ok && ocol + 7 < p.n_valid) {
+                *(uint4*)(base + (size_t)orow * p.ldc + ocol) = val;
+              } else {
+                const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                  if (ocol + k < p.n_valid) ((uint16_t*)base)[(size_t)orow * p.ldc + ocol + k] = (uint16_t)(w[k >> 1] >> ((k & 1) * 16));
+              }
+            }
+          }
+      }
+    };
+
+    store_wave(p.C);
+    if (SPLIT && MODE == MODE_SYRK2) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] -= bf16_to_f32(bf16_bits(acc[i][j][e]));
+      __builtin_amdgcn_sched_barrier(0);
+      store_wave(p.C2);
+    }
+    return;
+  }
+
+  // ---- block-cooperative epilogue for the diagonal tiles of a symmetric product (the upper half is
+  // reflected across waves so that the product is bit-symmetric)
 
   // 1. fold the addend into the accumulators: acc <- alpha*acc + beta*E (SYRK2), acc + alpha*E (BX), alpha*acc (SYRK)
   if (MODE != MODE_SYRK) {
