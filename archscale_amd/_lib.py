@@ -18,6 +18,7 @@ from .build import LIB_PATH
 DTYPE_BF16, DTYPE_F32 = 0, 1
 EPS_ADD, EPS_CLAMP = 0, 1
 PREC_BF16, PREC_BF16_BSPLIT = 0, 1
+ALGO_ADAMW, ALGO_LION = 0, 1
 NS_CAST_INPUT_FIRST = 1
 CHUNK_ELEMS = 8192
 ABI_VERSION = 1
@@ -28,7 +29,10 @@ PRE_ITEM = np.dtype(
      ("g_dtype", "<i4"), ("m_dtype", "<i4"), ("u_dtype", "<i4"), ("w_dtype", "<i4")], align=True)
 POST_ITEM = np.dtype(
     [("w", "<u8"), ("u", "<u8"), ("numel", "<i8"), ("lr_ratio", "<f4"), ("w_dtype", "<i4")], align=True)
-assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32
+SCALAR_ITEM = np.dtype(
+    [("w", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("numel", "<i8"),
+     ("w_dtype", "<i4"), ("g_dtype", "<i4"), ("m_dtype", "<i4"), ("v_dtype", "<i4")], align=True)
+assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32 and SCALAR_ITEM.itemsize == 56
 
 
 class NsProblem(ctypes.Structure):
@@ -66,6 +70,10 @@ _SIGNATURES = {
     "muon_profile_collect": (ctypes.c_int, [
         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_double),
         ctypes.POINTER(ctypes.c_double), ctypes.c_int]),
+    "muon_scalar_update": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_void_p]),
     "muon_calibration_copy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_syrk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
     "muon_syrk": (ctypes.c_int, [

@@ -2,6 +2,7 @@
 // workspace carving and the launch sequence of one Newton-Schulz call.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <math.h>
 #include <stdlib.h>
 
 #include <algorithm>
@@ -364,6 +365,23 @@ int muon_syrk(const void* a_dev, int64_t a_batch_stride, int lda, const void* c_
   e = launch_ns_gemm(tile, c_dev ? MODE_SYRK2 : MODE_SYRK, false, false, g, stream);
   if (e != hipSuccess) return (int)e;
   return (int)launch_unpad_copy(Dp, (long)Np * Np, Np, d_dev, d_batch_stride, ldd, batch, n, n, stream);
+}
+
+int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                       int algo, int hyperball, float lr, float beta1, float beta2, float lr_wd, float eps, int step,
+                       int cautious, float* scratch_dev, void* stream) {
+  if (n_items == 0) return 0;
+  if (!items_dev || !prefix_dev || n_items < 0 || total_chunks < n_items || step < 1) return MUON_E_ARG;
+  if (algo != MUON_ALGO_ADAMW && algo != MUON_ALGO_LION) return MUON_E_ARG;
+  if (hyperball && (algo != MUON_ALGO_ADAMW || !scratch_dev || ((uintptr_t)scratch_dev & 7))) return MUON_E_ARG;
+  ScalarHyper h;
+  h.lr = lr; h.lr_wd = lr_wd; h.eps = eps;
+  h.w1 = 1.f - beta1; h.w2 = 1.f - beta2;
+  h.bias1 = (float)(1.0 - pow((double)beta1, (double)step));
+  h.bias2_sqrt = (float)sqrt(1.0 - pow((double)beta2, (double)step));
+  h.cautious = cautious;
+  return (int)launch_scalar_update(items_dev, prefix_dev, n_items, total_chunks, algo, hyperball, h, scratch_dev,
+                                   (hipStream_t)stream);
 }
 
 int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {

@@ -12,6 +12,17 @@ enum { EPS_ADD = MUON_EPS_ADD, EPS_CLAMP = MUON_EPS_CLAMP };
 
 typedef muon_pre_item PreItem;
 typedef muon_post_item PostItem;
+typedef muon_scalar_item ScalarItem;
+
+enum { ALGO_ADAMW = MUON_ALGO_ADAMW, ALGO_LION = MUON_ALGO_LION };
+
+// hyper-parameters of the scalar updates, precomputed on the host
+struct ScalarHyper {
+  float lr, lr_wd, eps;
+  float w1, w2;            // 1 - beta1, 1 - beta2
+  float bias1, bias2_sqrt; // 1 - beta1^step, sqrt(1 - beta2^step)
+  int cautious;
+};
 
 struct MomentumCoef {
   float mm, mg, um, ug, l2;
@@ -39,6 +50,9 @@ hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n
 
 hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
                              float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream);
+
+hipError_t launch_scalar_update(const ScalarItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream);
 
 hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 

@@ -498,6 +498,140 @@ hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n
 }
 
 // ---------------------------------------------------------------------------
+// 5. AdamW / hyperball-AdamW / Lion for the non-matrix parameter groups (lit_gpt/optim/scalar_opts.py:118-443)
+//    phase 0: one-pass update (AdamW, Lion)
+//    phase 1: hyperball pass 1 - update M, V in place, reduce |x'|^2, |U|^2, <x',U> with U = M/denom/bias1
+//    phase 2: hyperball pass 2 - recompute U from the updated M, V and apply X <- alpha*x' + beta*U
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void load8_rt(const void* p, int dt, long i, float (&v)[8]) {
+  if (dt == DT_BF16) Elem<DT_BF16>::load8(p, i, v); else Elem<DT_F32>::load8(p, i, v);
+}
+__device__ __forceinline__ void store8_rt(void* p, int dt, long i, const float (&v)[8]) {
+  if (dt == DT_BF16) Elem<DT_BF16>::store8(p, i, v); else Elem<DT_F32>::store8(p, i, v);
+}
+__device__ __forceinline__ float load1_rt(const void* p, int dt, long i) {
+  return dt == DT_BF16 ? Elem<DT_BF16>::load1(p, i) : Elem<DT_F32>::load1(p, i);
+}
+__device__ __forceinline__ void store1_rt(void* p, int dt, long i, float v) {
+  if (dt == DT_BF16) Elem<DT_BF16>::store1(p, i, v); else Elem<DT_F32>::store1(p, i, v);
+}
+__device__ __forceinline__ float round_rt(float v, int dt) { return dt == DT_BF16 ? bf2f(f2bf(v)) : v; }
+
+// one element; returns the new weight, updates m, v (as rounded to their dtypes), accumulates sums
+template <int ALGO, int PHASE>
+__device__ __forceinline__ float scalar_elem(float x, float g, float& m, float& v, const ScalarHyper& h, int m_dt,
+                                             int v_dt, float alpha, float beta, float (&s)[3]) {
+  float u;
+  if (ALGO == ALGO_LION) {
+    const float gm = round_rt(g, m_dt);
+    const float t = m + h.w1 * (gm - m);                       // lerp(M, G, 1-beta1)
+    u = (t > 0.f) ? 1.f : ((t < 0.f) ? -1.f : 0.f);
+    m = round_rt(m + h.w2 * (gm - m), m_dt);                   // M <- lerp(M, G, 1-beta2)
+    const float xd = decayed(x, u, h.lr_wd, h.cautious);
+    return xd - h.lr * u;
+  }
+  if (PHASE != 2) {
+    const float gm = round_rt(g, m_dt);
+    m = round_rt(m + h.w1 * (gm - m), m_dt);                   // M <- lerp(M, G, 1-beta1)
+    const float g2 = round_rt(gm * gm, v_dt);
+    v = round_rt(v + h.w2 * (g2 - v), v_dt);                   // V <- lerp(V, G*G, 1-beta2)
+  }
+  const float dir = m / (sqrtf(v) / h.bias2_sqrt + h.eps);     // M / (sqrt(V/bias2) + eps)
+  if (PHASE == 0) {
+    const float xd = decayed(x, dir, h.lr_wd, h.cautious);
+    return xd - (h.lr / h.bias1) * dir;
+  }
+  u = dir / h.bias1;
+  const float xd = decayed(x, u, h.lr_wd, h.cautious);
+  if (PHASE == 1) { s[0] += xd * xd; s[1] += u * u; s[2] += xd * u; return x; }
+  return alpha * xd + beta * u;
+}
+
+template <int ALGO, int PHASE>
+__global__ void __launch_bounds__(EW_THREADS)
+scalar_update_kernel(const ScalarItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
+                     ScalarHyper h, float* __restrict__ partial, const float2* __restrict__ coef) {
+  __shared__ float red[12];
+  const int chunk = blockIdx.x;
+  const int ii = find_item(prefix, n_items, chunk);
+  const ScalarItem it = items[ii];
+  const long begin = (long)(chunk - prefix[ii]) * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
+  const bool has_v = ALGO == ALGO_ADAMW;
+  const bool vec_ok = aligned16(it.w) && aligned16(it.g) && aligned16(it.m) && (!has_v || aligned16(it.v)) &&
+                      (it.numel % EW_VEC == 0);
+  float alpha = 1.f, beta = 0.f;
+  if (PHASE == 2) { const float2 c = coef[ii]; alpha = c.x; beta = c.y; }
+  float s[3] = {0.f, 0.f, 0.f};
+  if (vec_ok) {
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float x[8], g[8], m[8], v[8];
+        load8_rt(it.w, it.w_dtype, i, x);
+        load8_rt(it.m, it.m_dtype, i, m);
+        if (PHASE != 2) load8_rt(it.g, it.g_dtype, i, g);
+        if (has_v) load8_rt(it.v, it.v_dtype, i, v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if (PHASE == 2) g[k] = 0.f;
+          if (!has_v) v[k] = 0.f;
+          x[k] = scalar_elem<ALGO, PHASE>(x[k], g[k], m[k], v[k], h, it.m_dtype, it.v_dtype, alpha, beta, s);
+        }
+        if (PHASE != 1) store8_rt(it.w, it.w_dtype, i, x);
+        if (PHASE != 2) {
+          store8_rt(it.m, it.m_dtype, i, m);
+          if (has_v) store8_rt(it.v, it.v_dtype, i, v);
+        }
+      }
+    }
+  } else {
+    for (long i = begin + threadIdx.x; i < end; i += EW_THREADS) {
+      float x = load1_rt(it.w, it.w_dtype, i), m = load1_rt(it.m, it.m_dtype, i);
+      float g = PHASE != 2 ? load1_rt(it.g, it.g_dtype, i) : 0.f;
+      float v = has_v ? load1_rt(it.v, it.v_dtype, i) : 0.f;
+      x = scalar_elem<ALGO, PHASE>(x, g, m, v, h, it.m_dtype, it.v_dtype, alpha, beta, s);
+      if (PHASE != 1) store1_rt(it.w, it.w_dtype, i, x);
+      if (PHASE != 2) {
+        store1_rt(it.m, it.m_dtype, i, m);
+        if (has_v) store1_rt(it.v, it.v_dtype, i, v);
+      }
+    }
+  }
+  if (PHASE == 1) {
+    block_reduce<3>(s, red);
+    if (threadIdx.x == 0) {
+      partial[(size_t)chunk * 3 + 0] = s[0];
+      partial[(size_t)chunk * 3 + 1] = s[1];
+      partial[(size_t)chunk * 3 + 2] = s[2];
+    }
+  }
+}
+
+hipError_t launch_scalar_update(const ScalarItem* items, const int32_t* prefix, int n_items, int total_chunks,
+                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream) {
+  if (total_chunks <= 0) return hipSuccess;
+  dim3 grid(total_chunks), block(EW_THREADS);
+  if (algo == ALGO_LION) {
+    hipLaunchKernelGGL((scalar_update_kernel<ALGO_LION, 0>), grid, block, 0, stream, items, prefix, n_items, h,
+                       (float*)nullptr, (const float2*)nullptr);
+  } else if (!hyperball) {
+    hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 0>), grid, block, 0, stream, items, prefix, n_items, h,
+                       (float*)nullptr, (const float2*)nullptr);
+  } else {
+    float* partial = scratch;
+    float2* coef = (float2*)(scratch + (size_t)3 * total_chunks + ((total_chunks & 1) ? 1 : 0));
+    hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 1>), grid, block, 0, stream, items, prefix, n_items, h,
+                       partial, (const float2*)nullptr);
+    hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), block, 0, stream, prefix, partial, h.lr, h.eps, coef);
+    hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 2>), grid, block, 0, stream, items, prefix, n_items, h,
+                       (float*)nullptr, (const float2*)coef);
+  }
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // plain copy of known size: calibrates the HBM byte counters (FETCH_SIZE / WRITE_SIZE) of a profiling run
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)

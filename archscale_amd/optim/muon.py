@@ -281,6 +281,7 @@ class Muon(Optimizer):
         self._muonh_per_matrix = muonh_per_matrix
         self._ns_workspace_limit = int(ns_workspace_limit)
         self._plans: Dict[int, Tuple[Tuple, _GroupPlan]] = {}
+        self._scalar_plans: dict = {}
         #: when set to a list, every phase of a muon group step appends (name, start_event, stop_event)
         self.phase_events: Optional[list] = None
 
@@ -439,9 +440,11 @@ class Muon(Optimizer):
         if not params:
             return
         moms = [self._get_or_initialize_state(p, "lion")["momentum"] for p in params]
+        grads = [g if g.is_contiguous() else g.contiguous() for g in to_local([p.grad for p in params])]
         scalar_opts.lion_update_foreach(
-            to_local(params), to_local([p.grad for p in params]), to_local(moms), float(group["lr"]),
-            float(group["beta1"]), float(group["beta2"]), float(group["weight_decay"]), bool(group["cautious_wd"]))
+            to_local(params), grads, to_local(moms), float(group["lr"]),
+            float(group["beta1"]), float(group["beta2"]), float(group["weight_decay"]), bool(group["cautious_wd"]),
+            key=("lion", tuple(id(p) for p in params)), cache=self._scalar_plans)
 
     def _adamw_group_step(self, group: dict) -> None:
         params = [p for p in group["params"] if p.grad is not None]
@@ -458,8 +461,10 @@ class Muon(Optimizer):
         for plist, fn in ((ball, scalar_opts.hyperball_adamw_update_foreach), (flat, scalar_opts.adamw_update_foreach)):
             if plist:
                 states = [self._get_or_initialize_state(p, "adamw") for p in plist]
-                fn(to_local(plist), to_local([p.grad for p in plist]), to_local([s["momentum"] for s in states]),
-                   to_local([s["variance"] for s in states]), *args)
+                grads = [g if g.is_contiguous() else g.contiguous() for g in to_local([p.grad for p in plist])]
+                fn(to_local(plist), grads, to_local([s["momentum"] for s in states]),
+                   to_local([s["variance"] for s in states]), *args,
+                   key=("adamw", tuple(id(p) for p in plist)), cache=self._scalar_plans)
 
 
 def zeropower_via_newtonschulz5(G: Tensor, epsilon: Union[float, Tensor] = 1e-7) -> Tensor:

@@ -1,90 +1,102 @@
-"""AdamW / hyperball-AdamW / Lion updates for the non-matrix parameter groups of ``Muon``.
+"""AdamW / hyperball-AdamW / Lion for the non-matrix parameter groups of ``Muon`` on MI355X.
 
-Counterpart of lit_gpt/optim/scalar_opts.py.  These groups (embeddings, norms, lm_head) are
-HBM-bound element-wise work next to the Muon path; they run as batched ``torch._foreach``
-device ops on the parameters' device - they are NOT part of the hand-written HIP path and
-are kept only so that one ``Muon`` object can drive a whole model, as in the reference.
+Counterpart of lit_gpt/optim/scalar_opts.py: the reference runs these groups (embeddings, norms, lm_head) as
+compiled ``torch._foreach`` graphs; here each group is ONE multi-tensor HIP launch (three for the hyperball
+variant: update moments + reduce norms, per-tensor coefficients, apply) through ``muon_scalar_update``.
 """
 from __future__ import annotations
 
-from typing import List
+from typing import Dict, List, Optional, Tuple
 
+import numpy as np
 import torch
 from torch import Tensor
 
-
-def _weight_decay_(X: List[Tensor], U: List[Tensor], lr: float, weight_decay: float, cautious_wd: bool) -> None:
-    """Plain ``X *= 1 - lr*wd`` or the cautious variant that decays only where ``X*U >= 0``
-    (scalar_opts.py:179-191 of the reference)."""
-    if cautious_wd:
-        keep = torch._foreach_mul(X, U)
-        torch._foreach_sign_(keep)
-        torch._foreach_add_(keep, 1)
-        torch._foreach_clamp_max_(keep, 1)
-        torch._foreach_mul_(keep, X)
-        torch._foreach_mul_(keep, lr * weight_decay)
-        torch._foreach_sub_(X, keep)
-    else:
-        torch._foreach_mul_(X, 1 - lr * weight_decay)
+from .. import _lib
 
 
-def _adam_moments_(G: List[Tensor], M: List[Tensor], V: List[Tensor], beta1: float, beta2: float) -> None:
-    g_m = [g.to(dtype=m.dtype) for g, m in zip(G, M)]
-    torch._foreach_lerp_(M, g_m, 1 - beta1)
-    g_sq = [(g * g).to(dtype=v.dtype) for g, v in zip(g_m, V)]
-    torch._foreach_lerp_(V, g_sq, 1 - beta2)
+class _ScalarPlan:
+    """Device item table of one list of parameters (uploaded again only when a data pointer changes)."""
+
+    def __init__(self, n: int, numels: List[int], device: torch.device, hyperball: bool):
+        from .muon import _DeviceTable  # local import: muon imports this module
+        chunk = _lib.CHUNK_ELEMS
+        self.items = np.zeros(n, dtype=_lib.SCALAR_ITEM)
+        prefix = np.zeros(n + 1, dtype=np.int32)
+        for i, ne in enumerate(numels):
+            prefix[i + 1] = prefix[i] + (ne + chunk - 1) // chunk
+        self.chunks = int(prefix[-1])
+        self.table = _DeviceTable(self.items.nbytes, device)
+        self.prefix_dev = torch.from_numpy(prefix).to(device)
+        n_scratch = _lib.lib().muon_muonh_scratch_floats(n, self.chunks) if hyperball else 0
+        self.scratch = torch.empty(max(n_scratch, 1), dtype=torch.float32, device=device)
+        self.sig: Optional[Tuple] = None
+
+    def refresh(self, X, G, M, V) -> None:
+        sig = tuple((x.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr() if v is not None else 0)
+                    for x, g, m, v in zip(X, G, M, V))
+        if sig == self.sig:
+            return
+        for row, x, g, m, v in zip(self.items, X, G, M, V):
+            row["w"], row["g"], row["m"] = x.data_ptr(), g.data_ptr(), m.data_ptr()
+            row["v"] = v.data_ptr() if v is not None else 0
+            row["numel"] = x.numel()
+            row["w_dtype"], row["g_dtype"] = _lib.dtype_code(x.dtype), _lib.dtype_code(g.dtype)
+            row["m_dtype"] = _lib.dtype_code(m.dtype)
+            row["v_dtype"] = _lib.dtype_code(v.dtype) if v is not None else 0
+        self.table.upload(self.items)
+        self.sig = sig
 
 
-def _adam_direction(M: List[Tensor], V: List[Tensor], beta2: float, step: int, epsilon: float) -> List[Tensor]:
-    """M / (sqrt(V / bias2) + eps)."""
-    bias2_sqrt = (1 - beta2 ** step) ** 0.5
-    denom = torch._foreach_sqrt(V)
-    torch._foreach_div_(denom, bias2_sqrt)
-    torch._foreach_add_(denom, epsilon)
-    return torch._foreach_div(M, denom)
+#: plans of calls made without an owner's cache (direct use of the functions below)
+_plans: Dict[Tuple, _ScalarPlan] = {}
 
 
-def adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False) -> None:
-    """AdamW with bias correction (scalar_opts.py:118-198 of the reference)."""
+def _run(cache, key, algo: int, hyperball: bool, X: List[Tensor], G: List[Tensor], M: List[Tensor], V, lr: float, beta1: float,
+         beta2: float, weight_decay: float, step: int, epsilon: float, cautious_wd: bool) -> None:
     if not X:
         return
-    _adam_moments_(G, M, V, beta1, beta2)
-    direction = _adam_direction(M, V, beta2, step, epsilon)
-    _weight_decay_(X, direction, lr, weight_decay, cautious_wd)
-    torch._foreach_mul_(direction, lr / (1 - beta1 ** step))
-    torch._foreach_sub_(X, direction)
+    device = X[0].device
+    V = V if V is not None else [None] * len(X)
+    for t in (*X, *G, *M, *(v for v in V if v is not None)):
+        _lib.require_cuda(t, "an optimizer tensor")
+        if t.device != device:
+            raise ValueError("all tensors of a parameter group must live on one device")
+        if not t.is_contiguous():
+            raise ValueError("parameters, gradients and optimizer state must be contiguous")
+    struct = (key, algo, hyperball, tuple((tuple(x.shape), x.dtype, g.dtype, m.dtype) for x, g, m in zip(X, G, M)))
+    cache = _plans if cache is None else cache
+    plan = cache.get(struct)
+    if plan is None:
+        plan = _ScalarPlan(len(X), [x.numel() for x in X], device, hyperball)
+        cache[struct] = plan
+    with torch.cuda.device(device):
+        plan.refresh(X, G, M, V)
+        st = _lib.lib().muon_scalar_update(
+            plan.table.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(X), plan.chunks, algo, int(hyperball),
+            lr, beta1, beta2, lr * weight_decay, epsilon, max(int(step), 1), int(cautious_wd),
+            plan.scratch.data_ptr() if hyperball else 0, _lib.current_stream_ptr(device))
+    _lib.check(st, "muon_scalar_update")
 
 
-def hyperball_adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon,
-                                   cautious_wd=False) -> None:
-    """AdamW direction applied on the hypersphere: step of relative size ``lr`` along the bias-corrected
-    direction, then renormalisation to the tensor's previous Frobenius norm
-    (scalar_opts.py:254-377, 396-437 of the reference; the all-reduces drop out on one GPU)."""
-    if not X:
-        return
-    _adam_moments_(G, M, V, beta1, beta2)
-    U = _adam_direction(M, V, beta2, step, epsilon)
-    torch._foreach_div_(U, 1 - beta1 ** step)
-    _weight_decay_(X, U, lr, weight_decay, cautious_wd)
-    x_norms = torch._foreach_norm(X)
-    u_norms = torch._foreach_norm(U)
-    scales = [xn / un.clamp_min(epsilon) for xn, un in zip(x_norms, u_norms)]
-    torch._foreach_mul_(U, scales)
-    torch._foreach_mul_(U, lr)
-    torch._foreach_sub_(X, U)
-    new_norms = torch._foreach_norm(X)
-    torch._foreach_mul_(X, [xn / nn.clamp_min(epsilon) for xn, nn in zip(x_norms, new_norms)])
+def adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False, *, key=None, cache=None):
+    """AdamW with bias correction over a list of tensors (scalar_opts.py:118-198 of the reference)."""
+    _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_ADAMW, False, X, G, M, V, lr, beta1, beta2, weight_decay, step,
+         epsilon, cautious_wd)
 
 
-def lion_update_foreach(X, G, M, lr, beta1, beta2, weight_decay, cautious_wd=False) -> None:
-    """Lion: sign of the beta1-interpolated momentum, then momentum EMA with beta2
-    (scalar_opts.py:201-251 of the reference)."""
-    if not X:
-        return
-    g_m = [g.to(dtype=m.dtype) for g, m in zip(G, M)]
-    U = torch._foreach_lerp(M, g_m, 1 - beta1)
-    torch._foreach_sign_(U)
-    torch._foreach_lerp_(M, g_m, 1 - beta2)
-    _weight_decay_(X, U, lr, weight_decay, cautious_wd)
-    torch._foreach_mul_(U, lr)
-    torch._foreach_sub_(X, U)
+def hyperball_adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False, *,
+                                   key=None, cache=None):
+    """Adam direction applied on the hypersphere, per tensor (scalar_opts.py:254-377, 396-437 of the reference)."""
+    _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_ADAMW, True, X, G, M, V, lr, beta1, beta2, weight_decay, step,
+         epsilon, cautious_wd)
+
+
+def lion_update_foreach(X, G, M, lr, beta1, beta2, weight_decay, cautious_wd=False, *, key=None, cache=None):
+    """Lion over a list of tensors (scalar_opts.py:201-251 of the reference)."""
+    _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_LION, False, X, G, M, None, lr, beta1, beta2, weight_decay, 1, 0.0,
+         cautious_wd)
+
+
+def release_plans() -> None:
+    _plans.clear()

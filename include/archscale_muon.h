@@ -169,6 +169,31 @@ size_t muon_muonh_scratch_floats(int n_items, int total_chunks);
 int muon_update_muonh(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
                       float lr, float lr_wd, float eps, int cautious, float* scratch_dev, void* stream);
 
+/* ---- AdamW / hyperball-AdamW / Lion for the non-matrix groups of the same optimizer ----------------
+ * One multi-tensor launch (three for hyperball) over every parameter of a group, replacing the foreach graphs of
+ * lit_gpt/optim/scalar_opts.py:118-251 (adamw_update_foreach, lion_update_foreach) and 254-443 (hyperball AdamW:
+ * step of relative size lr along the bias-corrected Adam direction, then renormalisation to the previous norm).
+ *   AdamW:  M <- lerp(M, G, 1-beta1); V <- lerp(V, G*G, 1-beta2); dir = M / (sqrt(V / (1-beta2^step)) + eps);
+ *           W <- x' - lr / (1-beta1^step) * dir            (x' = weight-decayed W, plain or cautious)
+ *   Lion:   U = sign(lerp(M, G, 1-beta1)); M <- lerp(M, G, 1-beta2); W <- x' - lr * U
+ * scratch_dev: only for hyperball, muon_muonh_scratch_floats(n_items, total_chunks) floats.
+ */
+#define MUON_ALGO_ADAMW 0
+#define MUON_ALGO_LION 1
+
+typedef struct muon_scalar_item {
+  void* w;       /* weights, in place */
+  const void* g; /* gradient */
+  void* m;       /* first moment / momentum, in place */
+  void* v;       /* second moment (AdamW), in place; unused for Lion */
+  int64_t numel;
+  int32_t w_dtype, g_dtype, m_dtype, v_dtype;
+} muon_scalar_item;
+
+int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                       int algo, int hyperball, float lr, float beta1, float beta2, float lr_wd, float eps, int step,
+                       int cautious, float* scratch_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

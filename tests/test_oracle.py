@@ -284,3 +284,34 @@ def test_emerging_step(method):
         O.emerging_muon_step(torch.randn(4), torch.randn(4), torch.zeros(4), lr=0.1, beta=0.9, wd=0.0,
                              nesterov=False, wd_method=method, steps=5, scale_mode="spectral_mup",
                              extra_scale=1.0)
+
+
+# ---------------------------------------------------------------------------
+# scalar optimizers of the non-matrix groups (oracle/scalar_oracle.py)
+# ---------------------------------------------------------------------------
+def test_scalar_oracle_closed_forms():
+    from oracle import scalar_oracle as S
+    g = torch.randn(7, 5)
+    x0 = torch.randn(7, 5)
+    # AdamW, first step from zero moments: M/bias1 = g, sqrt(V/bias2) = |g|  =>  x <- x(1-lr wd) - lr g/(|g|+eps)
+    x, m, v = x0.clone(), torch.zeros(7, 5), torch.zeros(7, 5)
+    S.adamw_update_foreach([x], [g], [m], [v], 0.1, 0.9, 0.95, 0.5, 1, 1e-8)
+    assert torch.allclose(x, x0 * (1 - 0.05) - 0.1 * g / (g.abs() + 1e-8), atol=1e-6)
+    assert torch.allclose(m, 0.1 * g) and torch.allclose(v, 0.05 * g * g)
+    # Lion: update is -lr*sign(lerp), momentum is the beta2 EMA
+    x, m = x0.clone(), torch.full((7, 5), 0.3)
+    S.lion_update_foreach([x], [g], [m], 0.1, 0.9, 0.99, 0.0)
+    assert torch.allclose(x, x0 - 0.1 * torch.sign(0.9 * 0.3 + 0.1 * g), atol=1e-7)
+    assert torch.allclose(m, 0.99 * 0.3 + 0.01 * g, atol=1e-7)
+    # cautious decay only where x*u >= 0
+    x, m = torch.tensor([[1.0, -1.0]]), torch.zeros(1, 2)
+    S.lion_update_foreach([x], [torch.tensor([[1.0, 1.0]])], [m], 0.1, 0.9, 0.99, 0.5, cautious_wd=True)
+    assert torch.allclose(x, torch.tensor([[1.0 - 0.05 - 0.1, -1.0 - 0.1]]))
+    # hyperball AdamW: norm preserved, moves along -direction
+    x, m, v = x0.clone(), torch.zeros(7, 5), torch.zeros(7, 5)
+    S.hyperball_adamw_update_foreach([x], [g], [m], [v], 0.1, 0.9, 0.95, 0.0, 1, 1e-8)
+    assert x.norm().item() == pytest.approx(x0.norm().item(), rel=1e-5)
+    d = g / (g.abs() + 1e-8)
+    want = x0 - 0.1 * x0.norm() / d.norm() * d
+    want = want * x0.norm() / want.norm()
+    assert torch.allclose(x, want, atol=1e-5)
