@@ -20,6 +20,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "ns_gemm.h"
 
 namespace archscale {
@@ -122,19 +124,17 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const int KT = p.K / BK;
   const int KT_ALL = KSPLIT ? 2 * KT : KT;
 
-  auto issue = [&](int kt, int stage) {
+  // copy j (of JP + JQ per wave) of k-tile kt: one 1 KiB slab (8 rows x 128 B) straight into stage kt & 1
+  constexpr int NGL = JP + JQ;
+  auto gload = [&](int kt, int j) {
     const char* pb = Pb;
     int kk = kt;
     if (KSPLIT && kt >= KT) { pb = P2b; kk = kt - KT; }
     const uint32_t koff = (uint32_t)kk * ROW_BYTES;
-    char* sP = smem + stage * STAGE;
+    char* sP = smem + (kt & 1) * STAGE;
     char* sQ = sP + PBYTES;
-#pragma unroll
-    for (int j = 0; j < JP; ++j)
-      __builtin_amdgcn_global_load_lds((gptr_t)(pb + offP[j] + koff), (lptr_t)(sP + (wave * JP + j) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int j = 0; j < JQ; ++j)
-      __builtin_amdgcn_global_load_lds((gptr_t)(Qb + offQ[j] + koff), (lptr_t)(sQ + (wave * JQ + j) * 1024), 16, 0, 0);
+    if (j < JP) __builtin_amdgcn_global_load_lds((gptr_t)(pb + offP[j] + koff), (lptr_t)(sP + (wave * JP + j) * 1024), 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)(Qb + offQ[j - JP] + koff), (lptr_t)(sQ + (wave * JQ + (j - JP)) * 1024), 16, 0, 0);
   };
 
   f32x16 acc[FM][FN];
@@ -155,46 +155,102 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     rdQ[kk] = lds_chunk_off(wc0 + l32, 2 * kk + hi);
   }
 
-  // Operand fragments are double-buffered in registers: while the MFMAs of k-step kk run, the LDS reads of
-  // kk+1 are issued, one read slotted after each MFMA (the scheduler is pinned to that order below;
-  // left alone it serialises read -> wait -> MFMA and the matrix pipe idles on LDS latency).
+  // ---- main loop.  A k-tile is four k-steps of FM*FN MFMAs; the operand fragments of a k-step are
+  // double-buffered in registers.  Every memory instruction is pinned behind an MFMA of its own:
+  //   * an LDS fragment read of the NEXT k-step after each of the first FM+FN MFMAs of a k-step;
+  //   * the global->LDS copies of a k-tile spread over the MFMAs of COPY_PHASES k-steps.  Issued back to
+  //     back, the copies hold the wave until the texture unit has accepted all of them (about as long as
+  //     the MFMAs of half a k-tile), and nothing overlaps.
+  // The loop is rotated by one k-step: the barrier that publishes k-tile kt+1 sits between k-steps 2 and 3
+  // of k-tile kt, so the MFMAs of k-step 3 run over the first fragment reads of the new tile and over the
+  // first copies of k-tile kt+2 into the stage that the barrier has just freed.
+  constexpr int NMF = FM * FN, NRD = FM + FN;
+  constexpr int COPY_PHASES = 2;
+  constexpr int GPP = (NGL + COPY_PHASES - 1) / COPY_PHASES;
+  constexpr int G1 = GPP < NGL ? GPP : NGL, G2 = 2 * GPP < NGL ? 2 * GPP : NGL, G3 = 3 * GPP < NGL ? 3 * GPP : NGL;
+  static_assert(G1 == 4 || G1 == 8 || G1 == 16, "the first wait below is written for these counts");
   bf16x8 af[2][FM], bq[2][FN];
-  auto load_frags = [&](int buf, const char* sP, const char* sQ, int kk) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i) af[buf][i] = *(const bf16x8*)(sP + rdP[kk] + i * 32 * ROW_BYTES);
-#pragma unroll
-    for (int j = 0; j < FN; ++j) bq[buf][j] = *(const bf16x8*)(sQ + rdQ[kk] + j * 32 * ROW_BYTES);
+  auto fread = [&](int buf, const char* sP, const char* sQ, int kk, int r) {
+    if (r < FM) af[buf][r] = *(const bf16x8*)(sP + rdP[kk] + r * 32 * ROW_BYTES);
+    else bq[buf][r - FM] = *(const bf16x8*)(sQ + rdQ[kk] + (r - FM) * 32 * ROW_BYTES);
   };
-
-  issue(0, 0);
-  for (int kt = 0; kt < KT_ALL; ++kt) {
-    const int stage = kt & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies for `stage` have landed
-    __syncthreads();                                  // everyone's have; everyone is done reading the other stage
-    if (kt + 1 < KT_ALL) issue(kt + 1, stage ^ 1);
-    const char* sP = smem + stage * STAGE;
-    const char* sQ = sP + PBYTES;
-    load_frags(0, sP, sQ, 0);
+  // one k-step: MFMAs on fragment buffer CBUF (when COMPUTE), reads of k-step RKK of the stage at (rP, rQ)
+  // into buffer RBUF (when READ), copies [G0, G1) of k-tile gt
+  auto phase = [&](auto compute, auto read, auto cbuf_, auto rbuf_, const char* rP, const char* rQ, auto rkk_, int gt,
+                   auto g0_, auto g1_) {
+    constexpr bool COMPUTE = decltype(compute)::value, READ = decltype(read)::value;
+    constexpr int cbuf = decltype(cbuf_)::value, rbuf = decltype(rbuf_)::value, rkk = decltype(rkk_)::value;
+    constexpr int g0 = decltype(g0_)::value, g1 = decltype(g1_)::value;
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+    for (int q = 0; q < NMF; ++q) {
+      if (COMPUTE)
+        acc[q / FN][q % FN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cbuf][q / FN], bq[cbuf][q % FN], acc[q / FN][q % FN], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-      if (kk + 1 < 4) load_frags((kk + 1) & 1, sP, sQ, kk + 1);
+      const int g_lo = g0 + (q * (g1 - g0) + NMF - 1) / NMF, g_hi = g0 + ((q + 1) * (g1 - g0) + NMF - 1) / NMF;
+      if (READ && q < NRD) fread(rbuf, rP, rQ, rkk, q);
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bq[kk & 1][j], acc[i][j], 0, 0, 0);
-      if (kk + 1 < 4) {
-#pragma unroll
-        for (int q = 0; q < FM + FN; ++q) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-        }
-        if (FM * FN > FM + FN) __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
-      }
+      for (int g = 0; g < NGL; ++g)
+        if (g >= g_lo && g < g_hi) gload(gt, g);
       __builtin_amdgcn_sched_barrier(0);
     }
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using C1 = std::integral_constant<int, G1>;
+  using C2 = std::integral_constant<int, G2>;
+  using C3 = std::integral_constant<int, G3>;
+  using C4 = std::integral_constant<int, NGL>;
+  // k-steps 0..2 of k-tile kt (with the rest of the copies of kt+1), barrier, k-step 3 (with the first
+  // copies of kt+2).  COPY_REST / NEXT / COPY_FIRST: k-tiles kt+1 / kt+1 / kt+2 exist.
+  auto ktile = [&](int kt, auto copy_rest, auto next, auto copy_first) {
+    constexpr bool COPY_REST = decltype(copy_rest)::value, NEXT = decltype(next)::value, COPY_FIRST = decltype(copy_first)::value;
+    const char* sP = smem + (kt & 1) * STAGE;
+    const char* sQ = sP + PBYTES;
+    const char* nP = smem + ((kt + 1) & 1) * STAGE;
+    const char* nQ = nP + PBYTES;
+    if constexpr (COPY_REST) {
+      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I1{}, kt + 1, C1{}, C2{});
+      phase(Yes{}, Yes{}, I1{}, I0{}, sP, sQ, I2{}, kt + 1, C2{}, C3{});
+      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I3{}, kt + 1, C3{}, C4{});
+    } else {
+      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I1{}, 0, I0{}, I0{});
+      phase(Yes{}, Yes{}, I1{}, I0{}, sP, sQ, I2{}, 0, I0{}, I0{});
+      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I3{}, 0, I0{}, I0{});
+    }
+    if constexpr (NEXT) {
+      // this wave's copies of kt+1 have landed and its reads of kt are done; after the barrier that holds for all
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (COPY_FIRST) phase(Yes{}, Yes{}, I1{}, I0{}, nP, nQ, I0{}, kt + 2, I0{}, C1{});
+      else phase(Yes{}, Yes{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
+    } else {
+      phase(Yes{}, No{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
+    }
+  };
+
+#pragma unroll
+  for (int g = 0; g < NGL; ++g) gload(0, g);
+  if (KT_ALL > 1) {
+#pragma unroll
+    for (int g = 0; g < G1; ++g) gload(1, g);
+    // k-tile 0 has landed once at most the G1 younger copies are outstanding
+    if constexpr (G1 == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else if constexpr (G1 == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < NRD; ++r) fread(0, smem, smem + PBYTES, 0, r);
+  for (int kt = 0; kt + 2 < KT_ALL; ++kt) ktile(kt, Yes{}, Yes{}, Yes{});
+  if (KT_ALL > 1) ktile(KT_ALL - 2, Yes{}, Yes{}, No{});
+  ktile(KT_ALL - 1, No{}, No{}, No{});
 
   // ---- epilogue.  acc[i][j][e] of lane l is element
   //   rl = wr0 + i*32 + 8*(e/4) + 4*(l/32) + e%4  (row in the tile),   cl = wc0 + j*32 + l%32  (column)
