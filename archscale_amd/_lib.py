@@ -19,9 +19,11 @@ DTYPE_BF16, DTYPE_F32 = 0, 1
 EPS_ADD, EPS_CLAMP = 0, 1
 PREC_BF16, PREC_BF16_BSPLIT = 0, 1
 ALGO_ADAMW, ALGO_LION = 0, 1
+RETRACT_HARD, RETRACT_DYNAMIC = 0, 1
+SN_TRANSPOSED = 1
 NS_CAST_INPUT_FIRST = 1
 CHUNK_ELEMS = 8192
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 #: numpy layouts of muon_pre_item / muon_post_item (natural C alignment)
 PRE_ITEM = np.dtype(
@@ -32,7 +34,10 @@ POST_ITEM = np.dtype(
 SCALAR_ITEM = np.dtype(
     [("w", "<u8"), ("g", "<u8"), ("m", "<u8"), ("v", "<u8"), ("numel", "<i8"),
      ("w_dtype", "<i4"), ("g_dtype", "<i4"), ("m_dtype", "<i4"), ("v_dtype", "<i4")], align=True)
-assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32 and SCALAR_ITEM.itemsize == 56
+BALL_ITEM = np.dtype(
+    [("w", "<u8"), ("phi", "<u8"), ("sigma", "<u8"), ("ld_w", "<i8"), ("ld_phi", "<i8"), ("rows", "<i4"), ("cols", "<i4"),
+     ("radius", "<f4"), ("lr_ratio", "<f4"), ("w_dtype", "<i4"), ("reserved", "<i4")], align=True)
+assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32 and SCALAR_ITEM.itemsize == 56 and BALL_ITEM.itemsize == 64
 
 
 class NsProblem(ctypes.Structure):
@@ -41,6 +46,13 @@ class NsProblem(ctypes.Structure):
                 ("in_batch_stride", ctypes.c_int64), ("out_batch_stride", ctypes.c_int64),
                 ("in_dtype", ctypes.c_int32), ("in_ld", ctypes.c_int32), ("out_ld", ctypes.c_int32),
                 ("batch", ctypes.c_int32), ("rows", ctypes.c_int32), ("cols", ctypes.c_int32)]
+
+
+class SnProblem(ctypes.Structure):
+    """muon_sn_problem of include/archscale_muon.h."""
+    _fields_ = [("w_ptrs", ctypes.POINTER(ctypes.c_void_p)), ("sigma_out", ctypes.c_void_p),
+                ("dtype", ctypes.c_int32), ("ld", ctypes.c_int32), ("batch", ctypes.c_int32),
+                ("rows", ctypes.c_int32), ("cols", ctypes.c_int32), ("flags", ctypes.c_int32)]
 
 
 class MuonLibraryError(RuntimeError):
@@ -92,6 +104,12 @@ _SIGNATURES = {
     "muon_update_muonh": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
         ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+    "muon_spectral_norm_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(SnProblem), ctypes.c_int]),
+    "muon_spectral_norm": (ctypes.c_int, [
+        ctypes.POINTER(SnProblem), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_ball_apply": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int,
+        ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -16,7 +16,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_NAME = "libarchscale_muon.so"
 LIB_PATH = os.path.join(LIB_DIR, LIB_NAME)
-SOURCES = ["ns_gemm.hip", "elementwise.hip", "abi.hip"]
+SOURCES = ["ns_gemm.hip", "elementwise.hip", "spectral.hip", "abi.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -12,6 +12,7 @@
 #include "../../include/archscale_muon.h"
 #include "elementwise.h"
 #include "ns_gemm.h"
+#include "spectral.h"
 
 using namespace archscale;
 
@@ -382,6 +383,154 @@ int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_
   h.cautious = cautious;
   return (int)launch_scalar_update(items_dev, prefix_dev, n_items, total_chunks, algo, hyperball, h, scratch_dev,
                                    (hipStream_t)stream);
+}
+
+// ---- MuonBall -------------------------------------------------------------------------------------------
+namespace {
+struct SnPlan {
+  NsPlan pl;
+  size_t off_x, off_g, off_z, off_part, total;
+};
+SnPlan make_sn_plan(int batch, int rows, int cols) {
+  SnPlan s;
+  s.pl = make_plan(batch, rows, cols, MUON_PREC_BF16);
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = (size_t)round_up((long)(off + bytes), 256); return o; };
+  s.off_x = take((size_t)batch * s.pl.Mp * s.pl.Np * 2);
+  s.off_g = take((size_t)batch * s.pl.Mp * s.pl.Mp * 2);
+  s.off_z = take((size_t)2 * batch * s.pl.Mp * sizeof(float));
+  s.off_part = take((size_t)2 * batch * (s.pl.Mp / SN_ROWS) * 2 * sizeof(float));
+  s.total = off;
+  return s;
+}
+int check_sn_problem(const muon_sn_problem& q) {
+  if (!q.w_ptrs || !q.sigma_out) return MUON_E_ARG;
+  if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0 || q.ld < q.cols) return MUON_E_ARG;
+  if (q.dtype != MUON_DTYPE_BF16 && q.dtype != MUON_DTYPE_F32) return MUON_E_ARG;
+  if (q.flags & ~MUON_SN_TRANSPOSED) return MUON_E_ARG;
+  for (int b = 0; b < q.batch; ++b)
+    if (!q.w_ptrs[b]) return MUON_E_ARG;
+  return 0;
+}
+}  // namespace
+
+size_t muon_spectral_norm_workspace_bytes(const muon_sn_problem* problems_host, int n_problems) {
+  if (!problems_host || n_problems <= 0) return 0;
+  size_t total = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    const muon_sn_problem& q = problems_host[i];
+    if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return 0;
+    total += make_sn_plan(q.batch, q.rows, q.cols).total;
+  }
+  return total;
+}
+
+int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int steps, void* ws_dev, size_t ws_bytes,
+                       void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!problems_host || n_problems <= 0 || steps < 1 || !ws_dev) return MUON_E_ARG;
+  if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
+  // tall: the matrix meant (after MUON_SN_TRANSPOSED) has more rows than columns; use_t: its short-side-first copy is
+  // the transpose of the stored block
+  struct Prob { muon_sn_problem q; SnPlan sp; __bf16 *X, *G; float *z, *part; bool tall, use_t; };
+  std::vector<Prob> pr(n_problems);
+  size_t off = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    Prob& P = pr[i];
+    P.q = problems_host[i];
+    const int st = check_sn_problem(P.q);
+    if (st) return st;
+    P.sp = make_sn_plan(P.q.batch, P.q.rows, P.q.cols);
+    if ((double)P.sp.pl.Mp * P.sp.pl.Np * 2.0 >= 4294967296.0) return MUON_E_UNSUPPORTED;
+    if (off + P.sp.total > ws_bytes) return MUON_E_WORKSPACE;
+    char* ws = (char*)ws_dev + off;
+    off += P.sp.total;
+    P.X = (__bf16*)(ws + P.sp.off_x);
+    P.G = (__bf16*)(ws + P.sp.off_g);
+    P.z = (float*)(ws + P.sp.off_z);
+    P.part = (float*)(ws + P.sp.off_part);
+    const bool transposed = (P.q.flags & MUON_SN_TRANSPOSED) != 0;
+    P.tall = transposed ? P.q.cols > P.q.rows : P.q.rows > P.q.cols;
+    P.use_t = transposed != P.tall;
+  }
+  hipError_t e;
+  // bf16 copy of every matrix with its short side first, zero padded to the GEMM tile
+  for (const Prob& P : pr) {
+    const NsPlan& pl = P.sp.pl;
+    const long xs = (long)pl.Mp * pl.Np;
+    for (int b = 0; b < P.q.batch; ++b) {
+      if (!P.use_t)
+        e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, P.X + b * xs, xs,
+                          pl.Np, pl.Mp, pl.Np, nullptr, 0, 0, stream);
+      else
+        e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, nullptr, 0, 0,
+                          pl.Np, pl.Mp, P.X + b * xs, xs, pl.Np, stream);
+      if (e != hipSuccess) return (int)e;
+    }
+  }
+  // G = X X^T: problems of one tile size share launches
+  for (int tile : {256, 128}) {
+    GroupedGemmParams gp = {};
+    auto flush = [&]() -> hipError_t {
+      if (gp.n_groups == 0) return hipSuccess;
+      hipError_t err = launch_ns_gemm_grouped(tile, MODE_SYRK, false, false, gp, stream);
+      gp = GroupedGemmParams{};
+      return err;
+    };
+    for (const Prob& P : pr) {
+      const NsPlan& pl = P.sp.pl;
+      if (pl.tile != tile) continue;
+      GemmParams g = {};
+      g.batch = P.q.batch;
+      g.P = P.X; g.Q = P.X; g.strideP = g.strideQ = (long)pl.Mp * pl.Np; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
+      g.tilesM = g.tilesN = pl.Mp / pl.tile;
+      g.C = P.G; g.strideC = (long)pl.Mp * pl.Mp; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
+      const long tiles = ns_gemm_tiles(MODE_SYRK, g);
+      if (tiles > 0x7ffffff0L) return MUON_E_UNSUPPORTED;
+      if (gp.n_groups == MAX_GROUPS || tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L) {
+        if ((e = flush()) != hipSuccess) return (int)e;
+      }
+      gp.g[gp.n_groups] = g;
+      gp.tile_start[gp.n_groups + 1] = gp.tile_start[gp.n_groups] + (int)tiles;
+      ++gp.n_groups;
+    }
+    if ((e = flush()) != hipSuccess) return (int)e;
+  }
+  // the rounds: classes of one orientation share a launch sequence
+  for (int kind = 0; kind < 2; ++kind) {
+    SnParams sp = {};
+    auto flush = [&]() -> hipError_t {
+      if (sp.n == 0) return hipSuccess;
+      hipError_t err = launch_spectral_iterate(sp, steps, stream);
+      sp = SnParams{};
+      return err;
+    };
+    for (const Prob& P : pr) {
+      if ((int)P.tall != kind) continue;
+      const NsPlan& pl = P.sp.pl;
+      const long blocks = (long)P.q.batch * (pl.Mp / SN_ROWS);
+      if (blocks > 0x3ffffff0L) return MUON_E_UNSUPPORTED;
+      if (sp.n == SN_MAX_CLASSES || blocks + sp.blk_start[sp.n] > 0x3ffffff0L) {
+        if ((e = flush()) != hipSuccess) return (int)e;
+      }
+      SnClass& c = sp.c[sp.n];
+      c.X = P.X; c.G = P.G; c.z = P.z; c.part = P.part; c.sigma = P.q.sigma_out;
+      c.batch = P.q.batch; c.d = pl.m; c.d_p = pl.Mp; c.L_p = pl.Np; c.nblk = pl.Mp / SN_ROWS; c.tall = P.tall ? 1 : 0;
+      sp.blk_start[sp.n + 1] = sp.blk_start[sp.n] + (int)blocks;
+      ++sp.n;
+    }
+    if ((e = flush()) != hipSuccess) return (int)e;
+  }
+  return 0;
+}
+
+int muon_ball_apply(const muon_ball_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks, float lr,
+                    float decay, int retract_mode, float retract_step, float* log_out_dev, void* stream) {
+  if (n_items == 0) return 0;
+  if (!items_dev || !prefix_dev || n_items < 0 || total_chunks < n_items) return MUON_E_ARG;
+  if (retract_mode != MUON_RETRACT_HARD && retract_mode != MUON_RETRACT_DYNAMIC) return MUON_E_ARG;
+  return (int)launch_ball_apply(items_dev, prefix_dev, n_items, total_chunks, lr, decay, retract_mode, retract_step,
+                                log_out_dev, (hipStream_t)stream);
 }
 
 int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {

@@ -36,7 +36,7 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
                              int rows, int cols, float eps, int eps_mode, float* partial, float* scale,
                              hipStream_t stream);
 
-// D = bf16(scale*in) in the input's orientation and T = its transpose (T may be null), both zero-padded to
+// D = bf16(scale*in) in the input's orientation and T = its transpose (either may be null), both zero-padded to
 // d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).
 hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,

@@ -264,7 +264,7 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
       o[k] = f2bf(x * s);
       tile[tr + h * 32][tc + k] = o[k];
     }
-    if (r < d_rows && c < d_cols) {
+    if (D && r < d_rows && c < d_cols) {
       uint4 pk;
       pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
       pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);

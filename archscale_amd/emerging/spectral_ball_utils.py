@@ -1,8 +1,10 @@
-"""Matrix sign by Newton-Schulz with the polar-express coefficients
-(emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:37-74, 142-149), on the HIP path."""
+"""Matrix sign by Newton-Schulz with the polar-express coefficients, spectral norm by power iteration, retraction,
+radius and scale of the spectral-ball optimizers
+(emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:37-74, 142-212, 432-466), on the HIP path."""
 from __future__ import annotations
 
-from typing import List, Tuple
+import math
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -34,3 +36,92 @@ def msign(G: torch.Tensor, steps: int) -> torch.Tensor:
     if G.dtype != torch.float32:
         raise ValueError("Input tensor G must be in float32")
     return ns.newton_schulz(G, msign_schedule(steps), 1e-7, eps_mode="clamp", prec="bsplit", cast_input_first=False)
+
+
+# ---------------------------------------------------------------------------
+# spectral norm, retraction, radius and scale of the spectral-ball family
+# ---------------------------------------------------------------------------
+def spectral_norm(w: torch.Tensor, steps: int = 50) -> torch.Tensor:
+    """Top singular value of every matrix of ``w`` ([..., rows, cols], bf16 or fp32) by the vector sequence of the
+    reference's power iteration (spectral_ball_utils.py:151-166), on the HIP path: one Gram matrix on the matrix
+    cores, then ``steps`` rounds of one launch each. Returns fp32 of shape ``w.shape[:-2]``; no host sync."""
+    import ctypes
+
+    from .. import _lib
+    if w.ndim < 2:
+        raise ValueError("Input tensor must have at least 2 dimensions.")
+    if steps < 1:
+        raise ValueError(f"steps must be at least 1, got {steps}")
+    _lib.require_cuda(w, "spectral_norm input")
+    if w.dtype not in (torch.bfloat16, torch.float32):
+        w = w.to(torch.float32)
+    rows, cols = w.shape[-2:]
+    mats = w.reshape(-1, rows, cols)
+    if mats.stride(-1) != 1 or mats.stride(-2) < cols:
+        mats = mats.contiguous()
+    batch = mats.shape[0]
+    sigma = torch.empty(batch, dtype=torch.float32, device=w.device)
+    ptrs = (ctypes.c_void_p * batch)(*[mats[b].data_ptr() for b in range(batch)])
+    prob = (_lib.SnProblem * 1)()
+    q = prob[0]
+    q.w_ptrs, q.sigma_out = ctypes.cast(ptrs, ctypes.POINTER(ctypes.c_void_p)), sigma.data_ptr()
+    q.dtype, q.ld, q.batch, q.rows, q.cols = _lib.dtype_code(mats.dtype), mats.stride(-2), batch, rows, cols
+    L = _lib.lib()
+    ws = _lib.workspace(w.device, L.muon_spectral_norm_workspace_bytes(prob, 1), tag="sn")
+    with torch.cuda.device(w.device):
+        st = L.muon_spectral_norm(prob, 1, steps, ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(w.device))
+    _lib.check(st, "muon_spectral_norm")
+    return sigma.reshape(w.shape[:-2])
+
+
+@torch.no_grad()
+def power_iteration(w: torch.Tensor, steps: int = 50, eps: float = 1e-20):
+    """(sigma, u, v) like spectral_ball_utils.py:151-166 of the reference. ``sigma`` comes from the HIP path
+    (:func:`spectral_norm`); the singular vectors, which MuonBall does not use, are recovered with plain matrix-vector
+    products (``eps`` is unused, as in the reference)."""
+    sigma = spectral_norm(w, steps)
+    wb = w.to(torch.bfloat16)
+    v = torch.ones_like(wb[..., :1, :].transpose(-2, -1))
+    for _ in range(steps):
+        v = torch.nn.functional.normalize(wb.transpose(-2, -1) @ (wb @ v), dim=-2)
+    u = torch.nn.functional.normalize(wb @ v, dim=-2)
+    return sigma, u, v
+
+
+@torch.no_grad()
+def apply_retract(W: torch.Tensor, sigma: float, target_radius: float, mode: str = "hard", alpha: float = 0.05,
+                  current_lr: Optional[float] = None) -> float:
+    """Host-scalar retraction of one matrix, in place (spectral_ball_utils.py:168-212). MuonBall itself applies the
+    same factor on the device, fused into its update kernel, without reading sigma back."""
+    if mode == "hard":
+        if max(sigma, 0.0) + 1e-8 != target_radius:
+            W.mul_(target_radius / (max(sigma, 0.0) + 1e-8))
+        return 0.0
+    if mode == "dynamic":
+        bias = -1.0 if sigma > target_radius else 1.0
+        W.mul_(1.0 + (alpha * current_lr if current_lr is not None else alpha) * bias)
+        return bias
+    raise ValueError(f"Unknown retract mode: {mode}")
+
+
+def compute_target_radius(shape: tuple, radius_mode: str, current_weight: Optional[torch.Tensor] = None,
+                          radius_scaler: float = 1.0) -> float:
+    """'spectral_mup' -> sqrt(n_out/n_in) * scaler, 'identity' -> scaler (spectral_ball_utils.py:432-440)."""
+    if radius_mode == "spectral_mup":
+        n_out, n_in = shape
+        return radius_scaler * math.sqrt(n_out / n_in)
+    if radius_mode == "identity":
+        return radius_scaler * 1.0
+    raise ValueError(f"Invalid radius_mode: {radius_mode}. Must be 'spectral_mup' or 'identity'.")
+
+
+def get_spectral_ball_scale_factor(size_out: int, size_in: int, mode: str = "spectral") -> float:
+    """spectral_ball_utils.py:442-466: align_adamw_rms 0.2*max(out,in)^0.5; shape_scaling max(1,out/in)^0.5;
+    spectral_mup (out/in)^0.5."""
+    if mode == "shape_scaling":
+        return max(1, size_out / size_in) ** 0.5
+    if mode == "align_adamw_rms":
+        return 0.2 * max(size_out, size_in) ** 0.5
+    if mode == "spectral_mup":
+        return (size_out / size_in) ** 0.5
+    raise ValueError(f"Invalid mode for SpectralBall update scale factor: {mode}")

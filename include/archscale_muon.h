@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define MUON_ABI_VERSION 1
+#define MUON_ABI_VERSION 2
 
 /* element types of caller tensors */
 #define MUON_DTYPE_BF16 0
@@ -193,6 +193,55 @@ typedef struct muon_scalar_item {
 int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
                        int algo, int hyperball, float lr, float beta1, float beta2, float lr_wd, float eps, int step,
                        int cautious, float* scratch_dev, void* stream);
+
+/* ---- MuonBall: spectral norm by power iteration, retraction and update ---------------------------------
+ * muon_spectral_norm estimates the top singular value of every matrix of every shape class with the vector
+ * sequence of power_iteration (emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:151-166:
+ * v <- normalize(W^T (W v)) `steps` times from v = 1, sigma = |W v|), run on the Gram matrix of the short side
+ * (one SYRK on the matrix cores per call, then one launch per round over all matrices; fp32 vectors).
+ * A problem is one shape class: `batch` matrices rows x cols with leading dimension ld, given by a HOST array of
+ * device pointers (the parameters of a model are separate allocations); the matrix is read as bf16 (fp32 input is
+ * rounded first, as the reference does, :158).  sigma_out: device, `batch` floats per problem.
+ * MUON_SN_TRANSPOSED in flags: the matrix meant is the TRANSPOSE of the stored rows x cols block (the reference
+ * hands W_expert.t() to the iteration, muon_ball.py:441-485; before convergence the estimate depends on the side the
+ * all-ones start vector lives on).
+ */
+#define MUON_SN_TRANSPOSED 1
+typedef struct muon_sn_problem {
+  const void* const* w_ptrs; /* host array of `batch` device pointers */
+  float* sigma_out;          /* device */
+  int32_t dtype, ld, batch, rows, cols, flags;
+} muon_sn_problem;
+
+size_t muon_spectral_norm_workspace_bytes(const muon_sn_problem* problems_host, int n_problems);
+int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int steps, void* workspace_dev,
+                       size_t workspace_bytes, void* stream);
+
+/* muon_ball_apply: for every item (a strided rows x cols block of a weight tensor)
+ *   W <- f * decay * W - lr * lr_ratio * Phi
+ * decay = 1 - lr*wd (decoupled) or 1 - wd (independent) or 1 (emerging_optimizers/mixin.py:33-52, applied before the
+ * power iteration in the reference, orthogonalized_optimizer.py:184-190: sigma(decay*W) = decay*sigma(W));
+ * f = R / (max(sigma,0) + 1e-8) (MUON_RETRACT_HARD) or 1 + retract_step * bias, bias = -1 if sigma > R else +1
+ * (MUON_RETRACT_DYNAMIC; retract_step = alpha*lr) (spectral_ball_utils.py:168-212); Phi = msign(momentum) in bf16,
+ * lr_ratio = the shape scale factor (muon_ball.py:349-352, 636-637; p.add_(update, alpha=-lr) :228).
+ * log_out_dev (nullable): 2 floats per item, (sigma of the decayed weights, bias).
+ */
+#define MUON_RETRACT_HARD 0
+#define MUON_RETRACT_DYNAMIC 1
+
+typedef struct muon_ball_item {
+  void* w;            /* weights, in place */
+  const void* phi;    /* orthogonalised update, bf16 */
+  const float* sigma; /* device: spectral norm of this block's matrix BEFORE weight decay; null = no retraction (f = 1) */
+  int64_t ld_w, ld_phi;
+  int32_t rows, cols;
+  float radius;   /* target spectral norm R (compute_target_radius, spectral_ball_utils.py:432-440) */
+  float lr_ratio; /* get_spectral_ball_scale_factor (:442-466) */
+  int32_t w_dtype, reserved;
+} muon_ball_item;
+
+int muon_ball_apply(const muon_ball_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks, float lr,
+                    float decay, int retract_mode, float retract_step, float* log_out_dev, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), f"{name} is declared in the header but not exported"
     assert sorted(_lib.EXPORTED_SYMBOLS) == declared
-    assert handle.muon_abi_version() == 1
+    assert handle.muon_abi_version() == _lib.ABI_VERSION == 2
     assert b"success" in handle.muon_status_string(0)
     assert b"workspace" in handle.muon_status_string(-2)
 
