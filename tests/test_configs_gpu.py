@@ -148,3 +148,46 @@ def test_config5_moe_full_step(gpu_device):
         # two steps of 2e-2 each: the oracle chain and the GPU chain stay within the single-step bar of each other
         assert _rel(got, x2) <= W_TOL
         assert _rel(got, x2) < 0.3 * _rel(w0[(i, e)], x2)
+
+
+def test_config2_muon_ball_full_step(gpu_device):
+    """MuonBall over the depth-16 dense parameter set (112 matrices): 50 power-iteration rounds, hard retraction,
+    msign with the polar-express table. Sampled matrices against the CPU oracle, every matrix against the sphere."""
+    from archscale_amd.emerging import MuonBall
+    from oracle import muon_ball_oracle as B
+    layer = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (5632, 2048), (5632, 2048), (2048, 5632)]
+    g = torch.Generator(device=gpu_device).manual_seed(1241)
+    params, grads = [], []
+    for _ in range(16):
+        for s in layer:
+            params.append(torch.nn.Parameter((torch.randn(*s, generator=g, device=gpu_device) * 0.02).to(torch.bfloat16)))
+            grads.append((torch.randn(*s, generator=g, device=gpu_device) * 1e-3).to(torch.bfloat16))
+    for p, gr in zip(params, grads):
+        p.grad = gr
+    lr = 0.02
+    opt = MuonBall(params, lr=lr, momentum_beta=0.95, weight_decay=0.0, use_nesterov=True, power_iteration_steps=50,
+                   msign_steps=5)
+    sample = [1, 6, 4, 59]
+    w0 = {i: params[i].detach().cpu().clone() for i in sample}
+    opt.step()
+    torch.cuda.synchronize()
+    for i in sample:
+        x, m = w0[i].clone(), torch.zeros_like(w0[i])
+        B.muon_ball_step(x, grads[i].cpu().clone(), m, lr=lr, beta=0.95, wd=0.0, nesterov=True, wd_method="decoupled",
+                         radius_mode="spectral_mup", scale_mode="align_adamw_rms", power_iteration_steps=50, msign_steps=5,
+                         retract_mode="hard", retract_alpha=0.05, ns_storage="fp32", sigma_fn=B.power_iteration_fp64)
+        assert _rel(params[i].detach(), x) <= W_TOL
+        assert _rel(opt.state[params[i]]["momentum_buffer"], m) < 1e-2          # bf16 state
+    # every matrix: spectral norm R up to the size of the update, lr * scale * |msign| <= lr * 0.2 sqrt(max dim) * 1.2
+    for p in params[:14]:
+        rows, cols = p.shape
+        R = math.sqrt(rows / cols)
+        top = torch.linalg.matrix_norm(p.detach().float(), ord=2).item()
+        assert abs(top - R) <= lr * 0.2 * math.sqrt(max(rows, cols)) * 1.2 + 0.02 * R
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(3):
+        opt.step()
+    ev1.record()
+    torch.cuda.synchronize()
+    print(f"config 2 MuonBall: {ev0.elapsed_time(ev1) / 3:.1f} ms/step (50 power-iteration rounds, msign 5 steps)", flush=True)
