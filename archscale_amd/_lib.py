@@ -153,6 +153,13 @@ def check(status: int, what: str) -> None:
         raise MuonLibraryError(f"{what}: HIP error {status}: {msg}")
 
 
+def ns_bsplit_tail(t: int) -> int:
+    """MUON_NS_BSPLIT_TAIL(t) of the header."""
+    if not 0 <= t <= 255:
+        raise ValueError(f"bsplit_tail must be in 0..255, got {t}")
+    return t << 8
+
+
 def dtype_code(dt: torch.dtype) -> int:
     if dt == torch.bfloat16:
         return DTYPE_BF16

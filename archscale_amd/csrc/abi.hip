@@ -167,7 +167,10 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
   if (eps_mode != MUON_EPS_ADD && eps_mode != MUON_EPS_CLAMP) return MUON_E_ARG;
   if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT) return MUON_E_ARG;
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
-  const bool split = prec_mode == MUON_PREC_BF16_BSPLIT;
+  const bool split_any = prec_mode == MUON_PREC_BF16_BSPLIT;
+  const int split_tail = (flags >> 8) & 0xff;   // 0: every iteration keeps B as a hi+lo pair; t: only the last t
+  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | 0xff00)) return MUON_E_ARG;
+  bool split = split_any;
   const int cast_first = (flags & MUON_NS_CAST_INPUT_FIRST) ? 1 : 0;
 
   std::vector<NsProblem> pr(n_problems);
@@ -187,7 +190,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     P.Xt[0] = (__bf16*)(ws + P.pl.off_xt[0]); P.Xt[1] = (__bf16*)(ws + P.pl.off_xt[1]);
     P.A = (__bf16*)(ws + P.pl.off_a);
     P.Bh = (__bf16*)(ws + P.pl.off_bh);
-    P.Bl = split ? (__bf16*)(ws + P.pl.off_bl) : nullptr;
+    P.Bl = split_any ? (__bf16*)(ws + P.pl.off_bl) : nullptr;
     P.partial = (float*)(ws + P.pl.off_partial);
     P.scale = (float*)(ws + P.pl.off_scale);
     P.tall = P.q.rows > P.q.cols;
@@ -259,6 +262,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
   for (int it = 0; it < iters; ++it) {
     const float a = abc_host[3 * it], b = abc_host[3 * it + 1], c = abc_host[3 * it + 2];
     const bool last = it == iters - 1;
+    split = split_any && (split_tail == 0 || it >= iters - split_tail);
     // A = X X^T
     e = run_mode(MODE_SYRK, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;

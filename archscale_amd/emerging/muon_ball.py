@@ -24,6 +24,7 @@ import torch
 from torch.optim.optimizer import ParamsT
 
 from .. import _lib
+from ..optim import newton_schulz_hip as ns
 from ..optim.muon import _DeviceTable
 from .mixin import WeightDecayT, weight_decay_terms
 from .orthogonalized_optimizer import OrthogonalizedOptimizer, _Plan
@@ -386,7 +387,8 @@ class MuonBall(OrthogonalizedOptimizer):
             ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(plan.ns_probs, n_ns, pm))
             coeffs = msign_schedule(self.msign_steps)
             _lib.check(L.muon_ns_grouped(plan.ns_probs, n_ns, _lib.abc_array(coeffs), len(coeffs), 1e-7, _lib.EPS_CLAMP,
-                                         pm, 0, ws.data_ptr(), ws.numel(), stream), "muon_ns_grouped")
+                                         pm, _lib.ns_bsplit_tail(ns.BSPLIT_TAIL), ws.data_ptr(), ws.numel(), stream),
+                       "muon_ns_grouped")
             for i, pc in enumerate(plan.pieces):
                 if pc.gather is None:
                     continue

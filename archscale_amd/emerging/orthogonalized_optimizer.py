@@ -187,7 +187,7 @@ class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
                 coeffs, eps, eps_mode, prec, _ = recipe
                 for key in plan.classes:
                     ns.newton_schulz(plan.U[key], coeffs, eps, eps_mode=eps_mode, prec=prec, cast_input_first=False,
-                                     out=plan.O[key])
+                                     out=plan.O[key], bsplit_tail=ns.BSPLIT_TAIL)
                 _lib.check(L.muon_update_plain(plan.post_tab.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(local),
                                                plan.chunks, lr, lr_wd, 0, stream), "muon_update_plain")
                 return

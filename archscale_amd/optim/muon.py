@@ -404,7 +404,8 @@ class Muon(Optimizer):
         def run():
             nonlocal parts, used
             if parts:
-                ns.newton_schulz_grouped(parts, self._ns_coefficients, eps, prec=self._ns_precision, outs=parts)
+                ns.newton_schulz_grouped(parts, self._ns_coefficients, eps, prec=self._ns_precision, outs=parts,
+                                         bsplit_tail=ns.BSPLIT_TAIL)
             parts, used = [], 0
 
         for cls in classes:

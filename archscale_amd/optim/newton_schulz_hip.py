@@ -34,6 +34,11 @@ QUINTIC_SCHEDULE: Coeffs = (
 SIMPLE_ROW = (3.4445, -4.7750, 2.0315)
 
 _PREC = {"bf16": _lib.PREC_BF16, "bsplit": _lib.PREC_BF16_BSPLIT}
+#: iterations (counted from the end) that keep B as a hi+lo pair wherever this package asks for the split itself.
+#: Measured against fp32 runs on the same bf16 input (N(0,1), 256x2048 .. 2048x5632): constant-row table x5
+#: 1.1-1.3e-2 without the split, 7.7-8.3e-3 with the last 2, 6.0-6.8e-3 with the last 3 and with all 5; the
+#: polar-express table x5 8.1-9.2e-3 / 6.9-8.5e-3 / 5.7-7.4e-3 / 5.7-7.3e-3.
+BSPLIT_TAIL = 3
 _EPS = {"add": _lib.EPS_ADD, "clamp": _lib.EPS_CLAMP}
 
 
@@ -68,13 +73,15 @@ def newton_schulz(
     prec: str = "bf16",
     cast_input_first: bool = True,
     out: Optional[Tensor] = None,
+    bsplit_tail: int = 0,
 ) -> Tensor:
     """Orthogonalise every matrix of ``G`` (``[..., rows, cols]``, bf16 or fp32) with the quintic
     Newton-Schulz iteration ``X <- aX + (bA + cA^2)X, A = XX^T``, one ``(a, b, c)`` row per iteration.
 
     Returns a new bf16 tensor shaped like ``G`` (``G`` itself is not modified unless ``out is G``).
     ``prec="bsplit"`` keeps ``B = bA + cA^2`` as a bf16 hi+lo pair (about +13% work) and is what the
-    constant-coefficient table needs to stay within 1e-2 of an fp32 run.
+    constant-coefficient table needs to stay within 1e-2 of an fp32 run; ``bsplit_tail=t`` does so only in the
+    last ``t`` iterations (0 = all), whose rounding dominates the error of the result.
     """
     _lib.require_cuda(G, "Newton-Schulz input")
     if G.dtype not in (torch.bfloat16, torch.float32):
@@ -92,7 +99,7 @@ def newton_schulz(
     pm = _PREC[prec]
     nbytes = L.muon_ns_workspace_bytes(batch, rows, cols, pm)
     ws = _lib.workspace(G.device, nbytes)
-    flags = _lib.NS_CAST_INPUT_FIRST if cast_input_first else 0
+    flags = (_lib.NS_CAST_INPUT_FIRST if cast_input_first else 0) | _lib.ns_bsplit_tail(bsplit_tail)
     with torch.cuda.device(G.device):
         st = L.muon_ns_batched(
             Gv.data_ptr(), _lib.dtype_code(Gv.dtype), bstride, ld,
@@ -113,6 +120,7 @@ def newton_schulz_grouped(
     prec: str = "bf16",
     cast_input_first: bool = True,
     outs: Optional[Sequence[Tensor]] = None,
+    bsplit_tail: int = 0,
 ) -> Sequence[Tensor]:
     """Orthogonalise several batches of DIFFERENT shapes in one call: every product of the iteration is a
     single kernel launch over the tiles of all batches (15 GEMM launches in total for five iterations).
@@ -142,7 +150,7 @@ def newton_schulz_grouped(
     L = _lib.lib()
     pm = _PREC[prec]
     ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(probs, len(views), pm))
-    flags = _lib.NS_CAST_INPUT_FIRST if cast_input_first else 0
+    flags = (_lib.NS_CAST_INPUT_FIRST if cast_input_first else 0) | _lib.ns_bsplit_tail(bsplit_tail)
     with torch.cuda.device(device):
         st = L.muon_ns_grouped(probs, len(views), _lib.abc_array(coeffs), len(coeffs), _as_float(epsilon),
                                _EPS[eps_mode], pm, flags, ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(device))
@@ -167,7 +175,7 @@ newton_schulz_triton = newton_schulz_hip
 def zeropower_via_newtonschulz5_legacy(G: Tensor, steps: int = 5) -> Tensor:
     """Drop-in for lit_gpt/legacy_optim.py:187-213: constant (3.4445, -4.7750, 2.0315) row, eps 1e-7."""
     assert G.ndim >= 2
-    return newton_schulz(G, [SIMPLE_ROW] * steps, 1e-7, prec="bsplit")
+    return newton_schulz(G, [SIMPLE_ROW] * steps, 1e-7, prec="bsplit", bsplit_tail=BSPLIT_TAIL)
 
 
 # ---------------------------------------------------------------------------

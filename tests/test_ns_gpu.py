@@ -168,3 +168,30 @@ def test_errors(ns, gpu_device):
     with pytest.raises(MuonLibraryError):
         ns.newton_schulz(torch.zeros(8, 8))
     assert math.isfinite(1.0)
+
+
+def test_bsplit_tail(gpu_device):
+    """Keeping B as a hi+lo pair only in the last t iterations: t = iters is the full split bit for bit, t = 3 stays at
+    the accuracy of the full split for the constant-row table, and unknown flag bits are rejected."""
+    import archscale_amd.optim.newton_schulz_hip as H
+    from archscale_amd import _lib
+    g = torch.Generator().manual_seed(31)
+    G = torch.randn(3, 384, 1024, generator=g).to(torch.bfloat16)
+    Gd = G.to(gpu_device)
+    coeffs = O.coefficient_schedule("simple", 5)
+    full = H.newton_schulz(Gd, coeffs, 1e-7, prec="bsplit")
+    assert torch.equal(H.newton_schulz(Gd, coeffs, 1e-7, prec="bsplit", bsplit_tail=5), full)
+    assert torch.equal(H.newton_schulz(Gd, coeffs, 1e-7, prec="bsplit", bsplit_tail=9), full)
+    want = O.newton_schulz(G, coeffs, 1e-7, storage="fp32")
+    e_full, e3, e0 = (_rel(x, want) for x in (full, H.newton_schulz(Gd, coeffs, 1e-7, prec="bsplit", bsplit_tail=3),
+                                              H.newton_schulz(Gd, coeffs, 1e-7, prec="bf16")))
+    assert e3 <= 1e-2 and e3 <= 1.1 * e_full and e0 > e3
+    assert torch.equal(H.newton_schulz(Gd, coeffs, 1e-7, prec="bf16", bsplit_tail=3), H.newton_schulz(Gd, coeffs, 1e-7, prec="bf16"))
+    assert H.BSPLIT_TAIL == 3
+    with pytest.raises(ValueError):
+        _lib.ns_bsplit_tail(256)
+    ws = _lib.workspace(gpu_device, 1 << 20)
+    abc = _lib.abc_array(coeffs)
+    st = _lib.lib().muon_ns_batched(Gd.data_ptr(), 0, 384 * 1024, 1024, full.data_ptr(), 384 * 1024, 1024, 3, 384, 1024, abc, 5,
+                                    1e-7, 0, 1, 1 << 20, ws.data_ptr(), ws.numel(), 0)
+    assert st < 0
