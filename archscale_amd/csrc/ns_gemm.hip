@@ -583,11 +583,16 @@ static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
   auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL>;
-  static bool attr_set = false;  // idempotent; a benign race only repeats the call
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device
+  // (idempotent; a benign race only repeats the call)
+  static bool attr_set[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
+    e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    if (dev >= 0 && dev < 64) attr_set[dev] = true;
   }
   const long tiles = gp.tile_start[gp.n_groups];
   if (tiles <= 0) return hipSuccess;
