@@ -26,7 +26,7 @@ struct NsPlan {
   int m, n;      // short / long side of a matrix
   int Mp, Np;    // padded to the tile
   int cpm;       // norm chunks per matrix
-  size_t off_x[2], off_xt[2], off_a, off_bh, off_bl, off_partial, off_scale, total;
+  size_t off_xt[2], off_a, off_bh, off_bl, off_partial, off_scale, total;
 };
 
 int pick_tile(int m, int n) {
@@ -54,8 +54,8 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode) {
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = (size_t)round_up((long)(off + bytes), 256); return o; };
   const size_t xb = (size_t)batch * p.Mp * p.Np * 2, ab = (size_t)batch * p.Mp * p.Mp * 2;
-  p.off_x[0] = take(xb); p.off_xt[0] = take(xb);
-  p.off_x[1] = take(xb); p.off_xt[1] = take(xb);
+  p.off_xt[0] = take(xb);
+  p.off_xt[1] = take(xb);
   p.off_a = take(ab);
   p.off_bh = take(ab);
   p.off_bl = prec_mode == MUON_PREC_BF16_BSPLIT ? take(ab) : 0;
@@ -135,7 +135,7 @@ namespace {
 struct NsProblem {
   muon_ns_problem q;
   NsPlan pl;
-  __bf16 *X[2], *Xt[2], *A, *Bh, *Bl;
+  __bf16 *Xt[2], *A, *Bh, *Bl;   // Xt: the iterate as X^T, [b][Np][Mp] (long side first), ping-pong
   float *partial, *scale;
   bool tall;
 };
@@ -186,7 +186,6 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     if (off + P.pl.total > ws_bytes) return MUON_E_WORKSPACE;
     char* ws = (char*)ws_dev + off;
     off += P.pl.total;
-    P.X[0] = (__bf16*)(ws + P.pl.off_x[0]); P.X[1] = (__bf16*)(ws + P.pl.off_x[1]);
     P.Xt[0] = (__bf16*)(ws + P.pl.off_xt[0]); P.Xt[1] = (__bf16*)(ws + P.pl.off_xt[1]);
     P.A = (__bf16*)(ws + P.pl.off_a);
     P.Bh = (__bf16*)(ws + P.pl.off_bh);
@@ -203,7 +202,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     return (long)pr[a].pl.Mp * pr[a].pl.Np > (long)pr[b].pl.Mp * pr[b].pl.Np;
   });
 
-  // normalise; the input's own orientation goes to X (wide) or X^T (tall), its transpose to the other
+  // normalise into X^T (long side first): a wide input is transposed on the way, a tall one is copied as it is
   hipError_t e;
   for (int i = 0; i < n_problems; ++i) {
     const NsProblem& P = pr[i];
@@ -214,10 +213,10 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     if (e != hipSuccess) return (int)e;
     if (!P.tall)
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, P.scale, P.X[0], xs, pl.Np, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
+                        P.q.cols, P.scale, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
     else
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, P.scale, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, P.X[0], xs, pl.Np, stream);
+                        P.q.cols, P.scale, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream);
     if (e != hipSuccess) return (int)e;
   }
 
@@ -229,7 +228,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
       double fa = 0.0, fi = 0.0;
       auto flush = [&]() -> hipError_t {
         if (gp.n_groups == 0) return hipSuccess;
-        hipError_t err = timed_gemm(tile, mode, split && mode != MODE_SYRK, last && mode == MODE_BX, gp, stream, fa, fi);
+        hipError_t err = timed_gemm(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi);
         gp = GroupedGemmParams{};
         fa = fi = 0.0;
         return err;
@@ -263,12 +262,12 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     const float a = abc_host[3 * it], b = abc_host[3 * it + 1], c = abc_host[3 * it + 2];
     const bool last = it == iters - 1;
     split = split_any && (split_tail == 0 || it >= iters - split_tail);
-    // A = X X^T
-    e = run_mode(MODE_SYRK, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+    // A = X X^T, from X^T (K-major operand)
+    e = run_mode(MODE_SYRKT, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
-      g.P = P.X[cur]; g.Q = P.X[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
+      g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
@@ -301,8 +300,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
       g.E = P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
       g.alpha = a; g.beta = 0.f;
       if (!last) {
-        g.C = P.X[cur ^ 1]; g.strideC = xs; g.ldc = pl.Np;
-        g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;
+        g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {
         g.m_valid = pl.m; g.n_valid = pl.n;
         if (!P.tall) { g.C = (__bf16*)P.q.out; g.strideC = P.q.out_batch_stride; g.ldc = P.q.out_ld; }

@@ -5,7 +5,8 @@
 
 namespace archscale {
 
-enum { MODE_SYRK = 0, MODE_SYRK2 = 1, MODE_BX = 2 };
+// MODE_SYRKT: as MODE_SYRK, but P = Q is given K-major ([K][M] row-major, ldp = leading dimension; P == Q required)
+enum { MODE_SYRK = 0, MODE_SYRK2 = 1, MODE_BX = 2, MODE_SYRKT = 3 };
 
 // C[m][n] = sum_k P[m][k] * Q[n][k]; all leading dimensions / strides in elements.
 struct GemmParams {

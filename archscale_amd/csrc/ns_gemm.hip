@@ -65,7 +65,11 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr int PBYTES = BM * ROW_BYTES, QBYTES = BN * ROW_BYTES, STAGE = PBYTES + QBYTES;
   constexpr int JP = BM / 8 / NW, JQ = BN / 8 / NW;  // 8-row slabs (1 KiB) per wave
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must split over waves");
-  constexpr bool SYM = (MODE == MODE_SYRK || MODE == MODE_SYRK2);
+  // MODE_SYRKT is MODE_SYRK with the operand given K-major: P = Q = X^T stored [K][M] (leading dimension ldp), so the
+  // iteration needs no row-major copy of X at all; the MFMA fragments then come from LDS transpose reads
+  constexpr bool KMAJ = (MODE == MODE_SYRKT);
+  constexpr bool SYRK_PLAIN = (MODE == MODE_SYRK || MODE == MODE_SYRKT);   // alpha * product, no addend
+  constexpr bool SYM = (SYRK_PLAIN || MODE == MODE_SYRK2);
   // SPLIT means "B is a hi+lo pair": SYRK2 WRITES the pair, BX READS it as a second pass over K
   constexpr bool KSPLIT = SPLIT && MODE == MODE_BX;
 
@@ -102,23 +106,41 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   }
   const int R0 = ti * BM, C0 = tj * BN;
 
-  const char* Pb = (const char*)(p.P + (size_t)b * p.strideP + (size_t)R0 * p.ldp);
+  const char* Pb = KMAJ ? (const char*)(p.P + (size_t)b * p.strideP + R0)
+                        : (const char*)(p.P + (size_t)b * p.strideP + (size_t)R0 * p.ldp);
   const char* P2b = KSPLIT ? (const char*)(p.P2 + (size_t)b * p.strideP + (size_t)R0 * p.ldp) : nullptr;
-  const char* Qb = (const char*)(p.Q + (size_t)b * p.strideQ + (size_t)C0 * p.ldq);
+  const char* Qb = KMAJ ? (const char*)(p.Q + (size_t)b * p.strideQ + C0)
+                        : (const char*)(p.Q + (size_t)b * p.strideQ + (size_t)C0 * p.ldq);
 
   // per-lane byte offsets of the global chunks this lane copies (k-tile 0)
   uint32_t offP[JP], offQ[JQ];
+  if constexpr (!KMAJ) {
 #pragma unroll
-  for (int j = 0; j < JP; ++j) {
-    const int r = (wave * JP + j) * 8 + (lane >> 3);
-    const int src = (lane & 7) ^ ((r >> 1) & 7);
-    offP[j] = (uint32_t)r * (uint32_t)p.ldp * 2u + (uint32_t)src * 16u;
-  }
+    for (int j = 0; j < JP; ++j) {
+      const int r = (wave * JP + j) * 8 + (lane >> 3);
+      const int src = (lane & 7) ^ ((r >> 1) & 7);
+      offP[j] = (uint32_t)r * (uint32_t)p.ldp * 2u + (uint32_t)src * 16u;
+    }
 #pragma unroll
-  for (int j = 0; j < JQ; ++j) {
-    const int r = (wave * JQ + j) * 8 + (lane >> 3);
-    const int src = (lane & 7) ^ ((r >> 1) & 7);
-    offQ[j] = (uint32_t)r * (uint32_t)p.ldq * 2u + (uint32_t)src * 16u;
+    for (int j = 0; j < JQ; ++j) {
+      const int r = (wave * JQ + j) * 8 + (lane >> 3);
+      const int src = (lane & 7) ^ ((r >> 1) & 7);
+      offQ[j] = (uint32_t)r * (uint32_t)p.ldq * 2u + (uint32_t)src * 16u;
+    }
+  } else {
+    // K-major tile in LDS: 64 k-rows of BM*2 bytes; the 16-byte chunk c of row k sits at chunk c ^ ((k & 3) << 2), so
+    // that four consecutive k-rows of one 64-byte column segment cover all 64 banks (what a transpose read touches)
+    constexpr int CPRK = BM / 8;   // chunks per k-row
+#pragma unroll
+    for (int j = 0; j < JP; ++j) {
+      const int pidx = (wave * JP + j) * 64 + lane, k = pidx / CPRK, cpos = pidx % CPRK;
+      offP[j] = (uint32_t)k * (uint32_t)p.ldp * 2u + (uint32_t)((cpos ^ ((k & 3) << 2)) * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < JQ; ++j) {
+      const int pidx = (wave * JQ + j) * 64 + lane, k = pidx / CPRK, cpos = pidx % CPRK;
+      offQ[j] = (uint32_t)k * (uint32_t)p.ldq * 2u + (uint32_t)((cpos ^ ((k & 3) << 2)) * 16);
+    }
   }
 
   const int KT = p.K / BK;
@@ -130,11 +152,12 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     const char* pb = Pb;
     int kk = kt;
     if (KSPLIT && kt >= KT) { pb = P2b; kk = kt - KT; }
-    const uint32_t koff = (uint32_t)kk * ROW_BYTES;
+    const size_t koffP = KMAJ ? (size_t)kk * BK * p.ldp * 2 : (size_t)kk * ROW_BYTES;
+    const size_t koffQ = KMAJ ? (size_t)kk * BK * p.ldq * 2 : (size_t)kk * ROW_BYTES;
     char* sP = smem + (kt & 1) * STAGE;
     char* sQ = sP + PBYTES;
-    if (j < JP) __builtin_amdgcn_global_load_lds((gptr_t)(pb + offP[j] + koff), (lptr_t)(sP + (wave * JP + j) * 1024), 16, 0, 0);
-    else __builtin_amdgcn_global_load_lds((gptr_t)(Qb + offQ[j - JP] + koff), (lptr_t)(sQ + (wave * JQ + (j - JP)) * 1024), 16, 0, 0);
+    if (j < JP) __builtin_amdgcn_global_load_lds((gptr_t)(pb + offP[j] + koffP), (lptr_t)(sP + (wave * JP + j) * 1024), 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)(Qb + offQ[j - JP] + koffQ), (lptr_t)(sQ + (wave * JQ + (j - JP)) * 1024), 16, 0, 0);
   };
 
   f32x16 acc[FM][FN];
@@ -154,6 +177,24 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     rdP[kk] = lds_chunk_off(wr0 + l32, 2 * kk + hi);
     rdQ[kk] = lds_chunk_off(wc0 + l32, 2 * kk + hi);
   }
+  // K-major operands: a 16-lane group reads 4 k-rows x 16 columns with one LDS transpose read; lane s = 4e + a of the
+  // group points at columns 4a..4a+3 of row k0 + e and receives, as lane 4a' + b', the 4 k-values of column 4a' + b'.
+  // Two such reads (k0, k0 + 4) make the 8 k-values of an MFMA operand; k0 = 16*kk + 8*(lane/32) is added below.
+  int trP[FM], trQ[FN];
+  if constexpr (KMAJ) {
+    const int g = lane >> 4, s16 = lane & 15, e = s16 >> 2, a = s16 & 3;
+    const int krow = 8 * (g >> 1) + e;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const int m = wr0 + i * 32 + (g & 1) * 16 + 4 * a;
+      trP[i] = krow * (BM * 2) + (((m >> 3) ^ (e << 2)) << 4) + ((m & 7) << 1);
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      const int n = wc0 + j * 32 + (g & 1) * 16 + 4 * a;
+      trQ[j] = krow * (BN * 2) + (((n >> 3) ^ (e << 2)) << 4) + ((n & 7) << 1);
+    }
+  }
 
   // ---- main loop.  A k-tile is four k-steps of FM*FN MFMAs; the operand fragments of a k-step are
   // double-buffered in registers.  Every memory instruction is pinned behind an MFMA of its own:
@@ -170,9 +211,27 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr int G1 = GPP < NGL ? GPP : NGL, G2 = 2 * GPP < NGL ? 2 * GPP : NGL, G3 = 3 * GPP < NGL ? 3 * GPP : NGL;
   static_assert(G1 == 4 || G1 == 8 || G1 == 16, "the first wait below is written for these counts");
   bf16x8 af[2][FM], bq[2][FN];
+  // The transpose reads are inline assembly: the compiler makes the builtin wait for every outstanding global->LDS
+  // copy (vmcnt(0)) before each read.  Their results are therefore not tracked by the compiler; an explicit
+  // s_waitcnt lgkmcnt(0), fenced, precedes the first MFMA of every k-step.
+  auto tr8 = [&](const char* base, int pitch, int kk) {
+    unsigned long long lo, hi4;
+    const uint32_t a0 = (uint32_t)(uintptr_t)base + (uint32_t)(16 * kk * pitch);
+    const uint32_t a1 = a0 + (uint32_t)(4 * pitch);
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a0));
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi4) : "v"(a1));
+    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+    const u64x2 v = {lo, hi4};
+    return __builtin_bit_cast(bf16x8, v);
+  };
   auto fread = [&](int buf, const char* sP, const char* sQ, int kk, int r) {
-    if (r < FM) af[buf][r] = *(const bf16x8*)(sP + rdP[kk] + r * 32 * ROW_BYTES);
-    else bq[buf][r - FM] = *(const bf16x8*)(sQ + rdQ[kk] + (r - FM) * 32 * ROW_BYTES);
+    if constexpr (!KMAJ) {
+      if (r < FM) af[buf][r] = *(const bf16x8*)(sP + rdP[kk] + r * 32 * ROW_BYTES);
+      else bq[buf][r - FM] = *(const bf16x8*)(sQ + rdQ[kk] + (r - FM) * 32 * ROW_BYTES);
+    } else {
+      if (r < FM) af[buf][r] = tr8(sP + trP[r], BM * 2, kk);
+      else bq[buf][r - FM] = tr8(sQ + trQ[r - FM], BN * 2, kk);
+    }
   };
   // one k-step: MFMAs on fragment buffer CBUF (when COMPUTE), reads of k-step RKK of the stage at (rP, rQ)
   // into buffer RBUF (when READ), copies [G0, G1) of k-tile gt
@@ -181,6 +240,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     constexpr bool COMPUTE = decltype(compute)::value, READ = decltype(read)::value;
     constexpr int cbuf = decltype(cbuf_)::value, rbuf = decltype(rbuf_)::value, rkk = decltype(rkk_)::value;
     constexpr int g0 = decltype(g0_)::value, g1 = decltype(g1_)::value;
+    if constexpr (KMAJ && COMPUTE) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int q = 0; q < NMF; ++q) {
       if (COMPUTE)
@@ -326,7 +389,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     auto w_off = [&](int c, int r) { return c * WROW + ((((r >> 3) ^ sw(c)) & (RCH - 1)) << 4) + ((r & 7) << 1); };
     const int wrow0 = R0 + wr0, wcol0 = C0 + wc0;  // global origin of this wave's sub-tile
 
-    if (MODE != MODE_SYRK) {
+    if (!SYRK_PLAIN) {
       const char* Eb = (const char*)(p.E + (size_t)b * p.strideE + (size_t)wcol0 * p.lde + wrow0);
 #pragma unroll
       for (int t = 0; t < WSLABS; ++t) {
@@ -344,7 +407,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int r = i * 32 + 8 * g + 4 * hi;
-          if (MODE == MODE_SYRK) {
+          if (SYRK_PLAIN) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
           } else {
@@ -459,7 +522,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   // reflected across waves so that the product is bit-symmetric)
 
   // 1. fold the addend into the accumulators: acc <- alpha*acc + beta*E (SYRK2), acc + alpha*E (BX), alpha*acc (SYRK)
-  if (MODE != MODE_SYRK) {
+  if (!SYRK_PLAIN) {
     // E[C0 + cl][R0 + rl] -> S[cl][rl], two staged rows (1 KiB) per wave-wide copy
     const char* Eb = (const char*)(p.E + (size_t)b * p.strideE + (size_t)C0 * p.lde + R0);
 #pragma unroll
@@ -481,7 +544,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int rl = wr0 + i * 32 + 8 * g + 4 * hi;
-        if (MODE == MODE_SYRK) {
+        if (SYRK_PLAIN) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
         } else {
@@ -502,7 +565,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
         }
       }
     }
-  if (MODE != MODE_SYRK) __syncthreads();  // the addend image is consumed; LDS is free again
+  if (!SYRK_PLAIN) __syncthreads();  // the addend image is consumed; LDS is free again
 
   // stores the accumulators as bf16 to Cdst (row-major image) and to its transposed / mirrored image
   auto store_all = [&](__bf16* Cdst) {
@@ -574,7 +637,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 // launch
 // ---------------------------------------------------------------------------
 long ns_gemm_tiles(int mode, const GemmParams& p) {
-  const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2);
+  const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2 || mode == MODE_SYRKT);
   return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
 }
 
@@ -606,6 +669,8 @@ static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGem
   switch (mode) {
     case MODE_SYRK:
       return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false>(p, s);
+    case MODE_SYRKT:
+      return launch_one<BM, BN, WM, WN, MODE_SYRKT, false, false>(p, s);
     case MODE_SYRK2:
       return split ? launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s)
                    : launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false>(p, s);

@@ -174,7 +174,7 @@ def main():
         k = (r["tile"], r["mode"], r["split"], r["final"])
         d = by_kernel.setdefault(k, dict(n=0, ms=0.0, fa=0.0, fi=0.0))
         d["n"] += 1; d["ms"] += r["ms"]; d["fa"] += r["flops_algorithmic"]; d["fi"] += r["flops_issued"]
-    names = {0: "syrk", 1: "syrk2", 2: "bx"}
+    names = {0: "syrk", 1: "syrk2", 2: "bx", 3: "syrk"}
     kernels = []
     for (tile, mode, split, final), d in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ms"]):
         kernels.append({
@@ -197,8 +197,8 @@ def main():
     }
     if args.layers == N_LAYERS:
         roofline["traffic"] = measured_traffic(roofline["kernel"])
-    if dom_key[1] == 2:  # B (m^2), X^T read twice (operand + addend), X' and X'^T written: bf16
-        per = [(min(s) ** 2 + 4 * min(s) * max(s)) * 2.0 for s in shapes]
+    if dom_key[1] == 2:  # B (m^2), X^T read twice (operand + addend), X'^T written (X' too by the final launch): bf16
+        per = [(min(s) ** 2 + 3 * min(s) * max(s)) * 2.0 for s in shapes]
         roofline["algorithmic_bytes_per_launch"] = sum(per) * (4 if not dom_key[3] else 1) / dom["n"]
     gemm_ms = sum(d["ms"] for d in by_kernel.values())
     f_issued = sum(d["fi"] for d in by_kernel.values())

@@ -62,7 +62,7 @@ def test_workspace_and_flops_queries_need_no_gpu():
     assert L.muon_ns_workspace_bytes(0, 8, 8, 0) == 0
     small = L.muon_ns_workspace_bytes(1, 512, 2048, 0)
     split = L.muon_ns_workspace_bytes(1, 512, 2048, 1)
-    assert split - small >= 512 * 512 * 2 and small >= 4 * 512 * 2048 * 2 + 2 * 512 * 512 * 2
+    assert split - small >= 512 * 512 * 2 and small >= 2 * 512 * 2048 * 2 + 2 * 512 * 512 * 2
     assert L.muon_ns_workspace_bytes(1, 2048, 512, 0) == small            # orientation does not matter
     d, s, i = _lib.ns_flops(1, 512, 2048, 5, 0)
     assert d == pytest.approx(5 * (4 * 512 ** 2 * 2048 + 2 * 512 ** 3))
