@@ -1,14 +1,13 @@
-// Newton-Schulz GEMMs for gfx950 (CDNA4): one "NT" MFMA kernel, three epilogues.
+// Newton-Schulz GEMMs for gfx950 (CDNA4): one MFMA kernel, three epilogues.
 //
-// Every product of the quintic iteration  X <- aX + (bA + cA^2)X,  A = X X^T  is
-// written as  C[m][n] = sum_k P[m][k] * Q[n][k]  with BOTH operands K-contiguous:
-//   SYRK   A  = X  * X^T         P = Q = X   (m x n_long)      upper-triangle tiles, mirrored store
-//   SYRK2  B  = c*A*A + b*A      P = Q = A   (A symmetric)     upper-triangle tiles, mirrored store
-//   BX     X' = a*X + B*X        P = B (symmetric), Q = X^T    writes X' and X'^T
-// Keeping X and X^T side by side is what makes the third product K-contiguous too,
-// so all three share one inner loop (replaces ns_line_1/ns_line_2 and the cuBLAS
-// addmm of lit_gpt/optim/newton_schulz_triton.py:66-139, 181-266, 371-378 and the
-// bf16 SYRK of emerging_optimizers/triton_kernels/syrk.py:104-185).
+// The iteration  X <- aX + (bA + cA^2)X,  A = X X^T  keeps ONLY the transposed iterate X^T ([n_long][m]):
+//   SYRKT  A  = X  * X^T         P = Q = X^T, a K-MAJOR operand ([k][m]); fragments by LDS transpose reads
+//   SYRK2  B  = c*A*A + b*A      P = Q = A   (A symmetric, K-contiguous)
+//   BX     X' = a*X + B*X        P = B (symmetric), Q = X^T (K-contiguous); writes X'^T (and X' only for the caller)
+// SYRK and SYRK2 compute upper-triangle tiles and mirror them.  SYRK (P = Q = X, K-contiguous) is the stand-alone
+// symmetric rank-k product.  All modes share one main loop (replaces ns_line_1/ns_line_2 and the cuBLAS addmm of
+// lit_gpt/optim/newton_schulz_triton.py:66-139, 181-266, 371-378 and the bf16 SYRK of
+// emerging_optimizers/triton_kernels/syrk.py:104-185).
 //
 // Operands live in zero-padded workspace buffers whose extents are multiples of
 // the tile sizes, so the main loop has no bounds checks; only the FINAL epilogue
