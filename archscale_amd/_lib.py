@@ -55,6 +55,16 @@ class SnProblem(ctypes.Structure):
                 ("rows", ctypes.c_int32), ("cols", ctypes.c_int32), ("flags", ctypes.c_int32)]
 
 
+class MnsProblem(ctypes.Structure):
+    """muon_mns_problem of include/archscale_muon.h."""
+    _fields_ = [("g_ptrs", ctypes.POINTER(ctypes.c_void_p)), ("m_ptrs", ctypes.POINTER(ctypes.c_void_p)),
+                ("w_ptrs", ctypes.POINTER(ctypes.c_void_p)), ("out", ctypes.c_void_p),
+                ("out_batch_stride", ctypes.c_int64), ("out_ld", ctypes.c_int32),
+                ("g_dtype", ctypes.c_int32), ("m_dtype", ctypes.c_int32), ("w_dtype", ctypes.c_int32),
+                ("batch", ctypes.c_int32), ("rows", ctypes.c_int32), ("cols", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
 class MuonLibraryError(RuntimeError):
     """The HIP library is missing, has the wrong ABI, or a call into it failed."""
 
@@ -75,6 +85,11 @@ _SIGNATURES = {
     "muon_ns_grouped_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(NsProblem), ctypes.c_int, ctypes.c_int]),
     "muon_ns_grouped": (ctypes.c_int, [
         ctypes.POINTER(NsProblem), ctypes.c_int,
+        ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_momentum_ns_grouped": (ctypes.c_int, [
+        ctypes.POINTER(MnsProblem), ctypes.c_int,
+        ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float,
         ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_ns_flops": (None, [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 3),

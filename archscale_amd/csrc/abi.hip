@@ -59,7 +59,9 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode) {
   p.off_a = take(ab);
   p.off_bh = take(ab);
   p.off_bl = prec_mode == MUON_PREC_BF16_BSPLIT ? take(ab) : 0;
-  p.off_partial = take((size_t)batch * p.cpm * sizeof(float));
+  // norm partials: one per 8192-element chunk (separate norm pass) or one per 64x64 tile of the padded matrix (fused pass)
+  const size_t tiles64 = (size_t)(p.Mp / 64) * (p.Np / 64);
+  p.off_partial = take((size_t)batch * std::max((size_t)p.cpm, tiles64) * sizeof(float));
   p.off_scale = take((size_t)batch * sizeof(float));
   p.total = off;
   return p;
@@ -140,8 +142,8 @@ struct NsProblem {
   bool tall;
 };
 
-int check_problem(const muon_ns_problem& q) {
-  if (!q.in || !q.out) return MUON_E_ARG;
+int check_problem(const muon_ns_problem& q, bool no_input = false) {
+  if ((!q.in && !no_input) || !q.out) return MUON_E_ARG;
   if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return MUON_E_ARG;
   if (q.in_ld < q.cols || q.out_ld < q.cols) return MUON_E_ARG;
   if (q.in_dtype != MUON_DTYPE_BF16 && q.in_dtype != MUON_DTYPE_F32) return MUON_E_ARG;
@@ -160,8 +162,13 @@ size_t muon_ns_grouped_workspace_bytes(const muon_ns_problem* problems_host, int
   return total;
 }
 
-int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const float* abc_host, int iters, float eps,
-                    int eps_mode, int prec_mode, int flags, void* ws_dev, size_t ws_bytes, void* stream_) {
+namespace {
+// The grouped Newton-Schulz call.  With `fused` (one entry per problem) the operand is not read from problems[i].in:
+// the momentum update of the matrices listed there produces it (unnormalised; the first iteration's epilogues apply
+// the scale), see momentum_layout_kernel.
+int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem* fused, MomentumCoef mc, int n_problems,
+                    const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags, void* ws_dev,
+                    size_t ws_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   if (!problems_host || n_problems <= 0 || !abc_host || !ws_dev || iters <= 0) return MUON_E_ARG;
   if (eps_mode != MUON_EPS_ADD && eps_mode != MUON_EPS_CLAMP) return MUON_E_ARG;
@@ -178,7 +185,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
   for (int i = 0; i < n_problems; ++i) {
     NsProblem& P = pr[i];
     P.q = problems_host[i];
-    const int st = check_problem(P.q);
+    const int st = check_problem(P.q, fused != nullptr);
     if (st) return st;
     P.pl = make_plan(P.q.batch, P.q.rows, P.q.cols, prec_mode);
     // byte offsets inside one matrix are 32-bit in the GEMM loader
@@ -204,7 +211,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
 
   // normalise into X^T (long side first): a wide input is transposed on the way, a tall one is copied as it is
   hipError_t e;
-  for (int i = 0; i < n_problems; ++i) {
+  for (int i = 0; i < n_problems && !fused; ++i) {
     const NsProblem& P = pr[i];
     const NsPlan& pl = P.pl;
     const long xs = (long)pl.Mp * pl.Np;
@@ -217,6 +224,34 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     else
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
                         P.q.cols, P.scale, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream);
+    if (e != hipSuccess) return (int)e;
+  }
+  // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials
+  for (int i = 0; i < n_problems && fused; ++i) {
+    const NsProblem& P = pr[i];
+    const NsPlan& pl = P.pl;
+    const muon_mns_problem& f = fused[i];
+    const long xs = (long)pl.Mp * pl.Np;
+    const int d_rows = P.tall ? pl.Np : pl.Mp, d_cols = P.tall ? pl.Mp : pl.Np;   // padded extents of the matrix itself
+    const int tiles = (d_rows / 64) * (d_cols / 64);
+    for (int b0 = 0; b0 < P.q.batch; b0 += MOMLAY_MAX) {
+      MomLayoutParams mp = {};
+      mp.n_mats = std::min(MOMLAY_MAX, P.q.batch - b0);
+      mp.rows = P.q.rows; mp.cols = P.q.cols;
+      mp.g_dtype = f.g_dtype; mp.m_dtype = f.m_dtype; mp.w_dtype = f.w_dtype;
+      mp.transpose = P.tall ? 0 : 1;
+      mp.d_rows = d_rows; mp.d_cols = d_cols; mp.ldd = pl.Mp; mp.d_bstride = xs;
+      mp.dst = (uint16_t*)(P.Xt[0] + (size_t)b0 * xs);
+      mp.partial = P.partial + (size_t)b0 * tiles;
+      mp.c = mc;
+      for (int k = 0; k < mp.n_mats; ++k) {
+        mp.g[k] = f.g_ptrs[b0 + k];
+        mp.m[k] = f.m_ptrs[b0 + k];
+        mp.w[k] = f.w_ptrs ? f.w_ptrs[b0 + k] : nullptr;
+      }
+      if ((e = launch_momentum_layout(mp, stream)) != hipSuccess) return (int)e;
+    }
+    e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);
     if (e != hipSuccess) return (int)e;
   }
 
@@ -270,6 +305,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
       g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
+      g.scale = (fused && it == 0) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
@@ -299,6 +335,7 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
       g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
       g.E = P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
       g.alpha = a; g.beta = 0.f;
+      g.scale = (fused && it == 0) ? P.scale : nullptr;
       if (!last) {
         g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {
@@ -314,6 +351,37 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const 
     cur ^= 1;
   }
   return 0;
+}
+}  // namespace
+
+int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems, const float* abc_host, int iters, float eps,
+                    int eps_mode, int prec_mode, int flags, void* ws_dev, size_t ws_bytes, void* stream) {
+  return ns_grouped_impl(problems_host, nullptr, MomentumCoef{}, n_problems, abc_host, iters, eps, eps_mode, prec_mode,
+                         flags, ws_dev, ws_bytes, stream);
+}
+
+int muon_momentum_ns_grouped(const muon_mns_problem* problems_host, int n_problems, float c_mm, float c_mg, float c_um,
+                             float c_ug, float l2, const float* abc_host, int iters, float eps, int eps_mode,
+                             int prec_mode, int flags, void* ws_dev, size_t ws_bytes, void* stream) {
+  if (!problems_host || n_problems <= 0) return MUON_E_ARG;
+  if (flags & MUON_NS_CAST_INPUT_FIRST) return MUON_E_ARG;   // the update is always rounded to bf16 before its norm here
+  std::vector<muon_ns_problem> q(n_problems);
+  for (int i = 0; i < n_problems; ++i) {
+    const muon_mns_problem& f = problems_host[i];
+    if (!f.g_ptrs || !f.m_ptrs || (l2 != 0.f && !f.w_ptrs) || !f.out || f.batch <= 0) return MUON_E_ARG;
+    for (int d : {f.g_dtype, f.m_dtype})
+      if (d != MUON_DTYPE_BF16 && d != MUON_DTYPE_F32) return MUON_E_ARG;
+    if (l2 != 0.f && f.w_dtype != MUON_DTYPE_BF16 && f.w_dtype != MUON_DTYPE_F32) return MUON_E_ARG;
+    for (int b = 0; b < f.batch; ++b)
+      if (!f.g_ptrs[b] || !f.m_ptrs[b] || (l2 != 0.f && !f.w_ptrs[b])) return MUON_E_ARG;
+    q[i].in = nullptr; q[i].out = f.out;
+    q[i].in_batch_stride = 0; q[i].out_batch_stride = f.out_batch_stride;
+    q[i].in_dtype = MUON_DTYPE_BF16; q[i].in_ld = f.cols; q[i].out_ld = f.out_ld;
+    q[i].batch = f.batch; q[i].rows = f.rows; q[i].cols = f.cols;
+  }
+  const MomentumCoef mc = {c_mm, c_mg, c_um, c_ug, l2};
+  return ns_grouped_impl(q.data(), problems_host, mc, n_problems, abc_host, iters, eps, eps_mode, prec_mode, flags, ws_dev,
+                         ws_bytes, stream);
 }
 
 int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld, void* out_dev,

@@ -42,6 +42,26 @@ hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_b
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
                          void* T, long t_bstride, int ldt, hipStream_t stream);
 
+// momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
+constexpr int MOMLAY_MAX = 32;
+struct MomLayoutParams {
+  int n_mats, rows, cols;        // matrices of this launch, all rows x cols, contiguous
+  int g_dtype, m_dtype, w_dtype;
+  int transpose;                 // dst holds the transpose of the matrix (d_cols x d_rows) instead of the matrix
+  int d_rows, d_cols;            // extents of the matrix padded to multiples of 64 (the grid)
+  int ldd;                       // leading dimension of dst
+  long d_bstride;                // elements between consecutive matrices in dst
+  uint16_t* dst;                 // bf16
+  float* partial;                // [n_mats][(d_rows/64) * (d_cols/64)] sums of squares
+  MomentumCoef c;
+  const void* g[MOMLAY_MAX];
+  void* m[MOMLAY_MAX];
+  const void* w[MOMLAY_MAX];     // read only when c.l2 != 0
+};
+hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream);
+hipError_t launch_norm_scale_from_partials(const float* partial, int partials_per_mat, int batch, float eps, int eps_mode,
+                                           float* scale, hipStream_t stream);
+
 hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
                              int batch, int rows, int cols, hipStream_t stream);
 

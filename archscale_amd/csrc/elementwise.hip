@@ -121,9 +121,9 @@ __device__ __forceinline__ void momentum_range(const PreItem& it, long begin, lo
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           const float gm = Elem<MD>::round(gv[k]);            // G cast to M's dtype (muon.py:666)
-          const float mn = Elem<MD>::round(c.mm * mv[k] + c.mg * gm);
+          const float mn = Elem<MD>::round(fmaf(c.mm, mv[k], c.mg * gm));
           mv[k] = mn;
-          uv[k] = c.um * mn + c.ug * gm;
+          uv[k] = fmaf(c.um, mn, c.ug * gm);
         }
         Elem<MD>::store8(m, i, mv);
         Elem<UD>::store8(u, i, uv);
@@ -138,9 +138,9 @@ __device__ __forceinline__ void momentum_range(const PreItem& it, long begin, lo
         Elem<GD>::store1(const_cast<void*>(g), i, gv);
       }
       const float gm = Elem<MD>::round(gv);
-      const float mn = Elem<MD>::round(c.mm * Elem<MD>::load1(m, i) + c.mg * gm);
+      const float mn = Elem<MD>::round(fmaf(c.mm, Elem<MD>::load1(m, i), c.mg * gm));
       Elem<MD>::store1(m, i, mn);
-      Elem<UD>::store1(u, i, c.um * mn + c.ug * gm);
+      Elem<UD>::store1(u, i, fmaf(c.um, mn, c.ug * gm));
     }
   }
 }
@@ -320,6 +320,132 @@ hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_b
   else if (cast_first) ARCHSCALE_NL(DT_F32, true);
   else ARCHSCALE_NL(DT_F32, false);
 #undef ARCHSCALE_NL
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// 3b. momentum fused with the layout pass: M <- c_mm*M + c_mg*G, U = c_um*M + c_ug*G as in momentum_kernel, but U is
+//     never stored in the parameter's orientation: its bf16 rounding goes straight into the Newton-Schulz operand
+//     (the matrix as it is, or its transpose, zero-padded) UNNORMALISED, with per-tile sums of squares; the
+//     normalisation 1/(|U| + eps) is applied by the first iteration's GEMM epilogues.  One launch covers up to
+//     MOMLAY_MAX matrices of one shape (their tensors are separate allocations: pointers by value).
+// ---------------------------------------------------------------------------
+template <int GD, int MD>
+__device__ __forceinline__ void momlay_tile(const MomLayoutParams& p, int mat, int r0, int c0, uint16_t (&tile)[64][66],
+                                            float& sumsq) {
+  const char* g = (const char*)p.g[mat];
+  char* m = (char*)p.m[mat];
+  const void* w = p.w[mat];
+  const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
+  const bool vec = aligned16(g) && aligned16(m) && (p.cols % 8 == 0) && (p.c.l2 == 0.f || aligned16(w));
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = r0 + tr + h * 32, c = c0 + tc;
+    float uv[8];
+    if (r < p.rows && c + 7 < p.cols && vec) {
+      const long i = (long)r * p.cols + c;
+      float gv[8], mv[8];
+      Elem<GD>::load8(g, i, gv);
+      Elem<MD>::load8(m, i, mv);
+      if (p.c.l2 != 0.f) {
+        float wv[8];
+        if (p.w_dtype == DT_BF16) Elem<DT_BF16>::load8(w, i, wv); else Elem<DT_F32>::load8(w, i, wv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) gv[k] = Elem<GD>::round(gv[k] + p.c.l2 * wv[k]);
+        Elem<GD>::store8(const_cast<char*>(g), i, gv);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float gm = Elem<MD>::round(gv[k]);
+        const float mn = Elem<MD>::round(fmaf(p.c.mm, mv[k], p.c.mg * gm));
+        mv[k] = mn;
+        uv[k] = fmaf(p.c.um, mn, p.c.ug * gm);
+      }
+      Elem<MD>::store8(m, i, mv);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        uv[k] = 0.f;
+        if (r < p.rows && c + k < p.cols) {
+          const long i = (long)r * p.cols + c + k;
+          float gv = Elem<GD>::load1(g, i);
+          if (p.c.l2 != 0.f) {
+            const float wv = p.w_dtype == DT_BF16 ? Elem<DT_BF16>::load1(w, i) : Elem<DT_F32>::load1(w, i);
+            gv = Elem<GD>::round(gv + p.c.l2 * wv);
+            Elem<GD>::store1(const_cast<char*>(g), i, gv);
+          }
+          const float gm = Elem<MD>::round(gv);
+          const float mn = Elem<MD>::round(fmaf(p.c.mm, Elem<MD>::load1(m, i), p.c.mg * gm));
+          Elem<MD>::store1(m, i, mn);
+          uv[k] = fmaf(p.c.um, mn, p.c.ug * gm);
+        }
+      }
+    }
+    uint16_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      o[k] = f2bf(uv[k]);
+      const float x = bf2f(o[k]);
+      sumsq += x * x;
+      tile[tr + h * 32][tc + k] = o[k];
+    }
+    if (!p.transpose) {
+      uint4 pk;
+      pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
+      pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
+      *(uint4*)(p.dst + (size_t)mat * p.d_bstride + (size_t)r * p.ldd + c) = pk;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+momentum_layout_kernel(const MomLayoutParams p) {
+  __shared__ uint16_t tile[64][66];
+  __shared__ float red[4];
+  const int mat = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;   // tile of the padded source orientation (d_rows x d_cols)
+  float s[1] = {0.f};
+  const int key = (p.g_dtype << 1) | p.m_dtype;
+  switch (key) {
+    case 0: momlay_tile<DT_BF16, DT_BF16>(p, mat, r0, c0, tile, s[0]); break;
+    case 1: momlay_tile<DT_BF16, DT_F32>(p, mat, r0, c0, tile, s[0]); break;
+    case 2: momlay_tile<DT_F32, DT_BF16>(p, mat, r0, c0, tile, s[0]); break;
+    default: momlay_tile<DT_F32, DT_F32>(p, mat, r0, c0, tile, s[0]); break;
+  }
+  __syncthreads();
+  if (p.transpose) {
+    const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int c = c0 + tr + h * 32;   // row of the transposed image
+      const int r = r0 + tc;            // 8 consecutive columns of it
+      uint16_t o[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) o[k] = tile[tc + k][tr + h * 32];
+      uint4 pk;
+      pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
+      pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
+      *(uint4*)(p.dst + (size_t)mat * p.d_bstride + (size_t)c * p.ldd + r) = pk;
+    }
+  }
+  block_reduce<1>(s, red);
+  if (threadIdx.x == 0) p.partial[(size_t)mat * gridDim.x * gridDim.y + blockIdx.y * gridDim.x + blockIdx.x] = s[0];
+}
+
+hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream) {
+  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.d_rows % 64 || p.d_cols % 64 || p.d_rows / 64 > 65535 ||
+      p.rows > p.d_rows || p.cols > p.d_cols || p.rows < 1 || p.cols < 1)
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(momentum_layout_kernel, dim3(p.d_cols / 64, p.d_rows / 64, p.n_mats), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+// scale[b] from per-tile (or per-chunk) partial sums written by another kernel
+hipError_t launch_norm_scale_from_partials(const float* partial, int partials_per_mat, int batch, float eps, int eps_mode,
+                                           float* scale, hipStream_t stream) {
+  if (batch < 1 || partials_per_mat < 1) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(norm_scale_kernel, dim3(batch), dim3(EW_THREADS), 0, stream, partial, partials_per_mat, eps, eps_mode,
+                     scale);
   return hipGetLastError();
 }
 

@@ -29,6 +29,7 @@ struct GemmParams {
   long strideCt;
   int ldct;
   float alpha, beta;
+  const float* scale;    // per batch element, or null: SYRK / SYRKT multiply the product by scale^2, BX the result by scale
   int m_valid, n_valid;  // true extents for the bounds-checked final store
 };
 

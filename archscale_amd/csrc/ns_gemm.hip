@@ -330,7 +330,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr int CPRT = BN / 8;              // 16-byte chunks per staged row
   constexpr int PASSES = (BM * BN / 8) / NT;
   static_assert(BM * BN * 2 <= 2 * STAGE, "staging tile must fit in the operand stages");
-  const float alpha = p.alpha, beta = p.beta;
+  // optional per-matrix scale of the operand that was left out of it (deferred normalisation): the product of two
+  // such operands carries sc^2, a product with one of them (and its addend) carries sc
+  const float sc = p.scale ? p.scale[b] : 1.f;
+  const float alpha = SYRK_PLAIN ? p.alpha * sc * sc : p.alpha, beta = p.beta;
   const bool diag = SYM && (ti == tj);
   // S[cl][rl]: chunk index XOR cl, so the 32 lanes of an 8-byte access (32 different cl) spread over all banks
   auto s_off = [](int cl, int rl) { return cl * TPITCH + ((((rl >> 3) ^ cl) & (CPRT - 1)) << 4) + ((rl & 7) << 1); };
@@ -419,10 +422,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
               acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
               acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
             } else {
-              acc[i][j][4 * g + 0] += alpha * e0;
-              acc[i][j][4 * g + 1] += alpha * e1;
-              acc[i][j][4 * g + 2] += alpha * e2;
-              acc[i][j][4 * g + 3] += alpha * e3;
+              acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * sc;
+              acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * sc;
+              acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * sc;
+              acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * sc;
             }
           }
         }
@@ -556,10 +559,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
             acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
             acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
           } else {
-            acc[i][j][4 * g + 0] += alpha * e0;
-            acc[i][j][4 * g + 1] += alpha * e1;
-            acc[i][j][4 * g + 2] += alpha * e2;
-            acc[i][j][4 * g + 3] += alpha * e3;
+            acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * sc;
+            acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * sc;
+            acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * sc;
+            acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * sc;
           }
         }
       }

@@ -169,6 +169,9 @@ class _GroupPlan:
         n_scratch = _lib.lib().muon_muonh_scratch_floats(len(post_rows), self.post_chunks) if use_muonh else 0
         self.scratch = torch.empty(max(n_scratch, 1), dtype=torch.float32, device=device)
         self.ptr_sig: Optional[Tuple] = None
+        # fused momentum + Newton-Schulz call: one problem per (shape class, dtypes), matrices listed by pointer
+        self.fused_probs = None
+        self.fused_keep: List = []
 
     def refresh_pointers(self, grads: List[Tensor], moms: List[Tensor]) -> None:
         sig = tuple((p.data_ptr(), g.data_ptr(), m.data_ptr()) for p, g, m in zip(self.params, grads, moms))
@@ -191,6 +194,36 @@ class _GroupPlan:
         self.pre_tab.upload(self.pre)
         self.post_tab.upload(self.post)
         self.ptr_sig = sig
+        self._build_fused(grads, moms)
+
+    def _build_fused(self, grads: List[Tensor], moms: List[Tensor]) -> None:
+        """muon_mns_problem array: per shape class the (g, m, w) pointers of its matrices in the order of its U buffer.
+        A class whose tensors do not share one dtype triple is left to the unfused path (fused_probs = None)."""
+        import ctypes
+        per_class: Dict[Tuple[int, int], List[Tuple[int, int, int, Tuple]]] = {k: [] for k in self.classes}
+        for i, (p, g, m) in enumerate(zip(self.params, grads, moms)):
+            cls, first, nm = self.views[i]
+            per = cls.rows * cls.cols
+            for k in range(nm):
+                per_class[(cls.rows, cls.cols)].append((g.data_ptr() + k * per * g.element_size(),
+                                                        m.data_ptr() + k * per * m.element_size(),
+                                                        p.data_ptr() + k * per * p.element_size(),
+                                                        (g.dtype, m.dtype, p.dtype)))
+        probs = (_lib.MnsProblem * len(self.classes))()
+        keep = []
+        for q, (key, cls) in zip(probs, self.classes.items()):
+            rows = per_class[key]
+            if len({r[3] for r in rows}) != 1:
+                self.fused_probs = None
+                return
+            arrs = [(ctypes.c_void_p * len(rows))(*[r[j] for r in rows]) for j in range(3)]
+            keep.append(arrs)
+            q.g_ptrs, q.m_ptrs, q.w_ptrs = (ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p)) for a in arrs)
+            q.out, q.out_batch_stride, q.out_ld = cls.U.data_ptr(), cls.rows * cls.cols, cls.cols
+            gd, md, wd = rows[0][3]
+            q.g_dtype, q.m_dtype, q.w_dtype = _lib.dtype_code(gd), _lib.dtype_code(md), _lib.dtype_code(wd)
+            q.batch, q.rows, q.cols = len(rows), cls.rows, cls.cols
+        self.fused_probs, self.fused_keep = probs, keep
 
 
 class Muon(Optimizer):
@@ -205,6 +238,8 @@ class Muon(Optimizer):
       ns_coefficients   (a, b, c) rows, one per iteration (default: the reference's 5-row schedule)
       ns_precision      "bf16" or "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair)
       muonh_per_matrix  renormalise each matrix of a 3-D parameter on its own instead of the whole tensor
+      fuse_momentum     momentum and Newton-Schulz in one library call that never stores the bf16 update in the
+                        parameter's orientation (default; falls back to separate calls with a hook or a tight limit)
       ns_workspace_limit  upper bound in bytes for one batched Newton-Schulz workspace (larger classes
                           are processed in slices)
     """
@@ -230,6 +265,7 @@ class Muon(Optimizer):
         ns_precision: str = "bf16",
         muonh_per_matrix: bool = False,
         ns_workspace_limit: int = 48 << 30,
+        fuse_momentum: bool = True,
     ):
         if lr < 0.0:
             raise ValueError(f"Invalid learning rate: {lr}")
@@ -280,6 +316,7 @@ class Muon(Optimizer):
         self._ns_precision = ns_precision
         self._muonh_per_matrix = muonh_per_matrix
         self._ns_workspace_limit = int(ns_workspace_limit)
+        self._fuse_momentum = bool(fuse_momentum)
         self._plans: Dict[int, Tuple[Tuple, _GroupPlan]] = {}
         self._scalar_plans: dict = {}
         #: when set to a list, every phase of a muon group step appends (name, start_event, stop_event)
@@ -370,17 +407,18 @@ class Muon(Optimizer):
         with torch.cuda.device(device):
             plan.refresh_pointers(grads, moms)
             stream = _lib.current_stream_ptr(device)
-            # M <- mu*M + G ; U <- mu*M + G (nesterov) | M, in bf16       (muon.py:653-681)
-            with self._timed("momentum"):
-                _lib.check(L.muon_momentum(plan.pre_tab.dev.data_ptr(), plan.pre_prefix_dev.data_ptr(), len(local),
-                                           plan.pre_chunks, mu, 1.0, mu if nesterov else 1.0,
-                                           1.0 if nesterov else 0.0, 0.0, stream), "muon_momentum")
-            # U <- NS(U), one batched call per shape class                    (muon.py:821-838)
-            if self._newton_schulz_func is None:
-                with self._timed("newton_schulz"):
-                    self._orthogonalize_classes(list(plan.classes.values()), eps)
-            else:
-                self._orthogonalize_with_hook(plan, eps)
+            c_um, c_ug = (mu, 1.0) if nesterov else (1.0, 0.0)
+            if not self._momentum_and_ns_fused(plan, mu, c_um, c_ug, eps, stream):
+                # M <- mu*M + G ; U <- mu*M + G (nesterov) | M, in bf16       (muon.py:653-681)
+                with self._timed("momentum"):
+                    _lib.check(L.muon_momentum(plan.pre_tab.dev.data_ptr(), plan.pre_prefix_dev.data_ptr(), len(local),
+                                               plan.pre_chunks, mu, 1.0, c_um, c_ug, 0.0, stream), "muon_momentum")
+                # U <- NS(U), one batched call per shape class                    (muon.py:821-838)
+                if self._newton_schulz_func is None:
+                    with self._timed("newton_schulz"):
+                        self._orthogonalize_classes(list(plan.classes.values()), eps)
+                else:
+                    self._orthogonalize_with_hook(plan, eps)
             # weight update                                                   (muon.py:598-650)
             with self._timed("update_muonh" if self.use_muonh else "update_plain"):
                 if self.use_muonh:
@@ -392,6 +430,26 @@ class Muon(Optimizer):
                     _lib.check(L.muon_update_plain(plan.post_tab.dev.data_ptr(), plan.post_prefix_dev.data_ptr(),
                                                    len(plan.post_rows), plan.post_chunks, lr, lr * wd, int(cautious),
                                                    stream), "muon_update_plain")
+
+    def _momentum_and_ns_fused(self, plan: _GroupPlan, mu: float, c_um: float, c_ug: float, eps: float, stream) -> bool:
+        """Momentum and Newton-Schulz of the whole group in ONE library call in which the bf16 update goes straight
+        into the operand of the iteration (no separate store, norm pass and layout pass over it). Used with the
+        built-in Newton-Schulz when the workspace of all classes together fits the limit; returns False otherwise."""
+        if self._newton_schulz_func is not None or not self._fuse_momentum or plan.fused_probs is None:
+            return False
+        L = _lib.lib()
+        pm = _lib.PREC_BF16_BSPLIT if self._ns_precision == "bsplit" else _lib.PREC_BF16
+        n = len(plan.fused_probs)
+        need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in plan.fused_probs)
+        if need > self._ns_workspace_limit:
+            return False
+        ws = _lib.workspace(plan.device, need)
+        coeffs = self._ns_coefficients
+        with self._timed("momentum+newton_schulz"):
+            _lib.check(L.muon_momentum_ns_grouped(plan.fused_probs, n, mu, 1.0, c_um, c_ug, 0.0, _lib.abc_array(coeffs),
+                                                  len(coeffs), eps, _lib.EPS_ADD, pm, _lib.ns_bsplit_tail(ns.BSPLIT_TAIL),
+                                                  ws.data_ptr(), ws.numel(), stream), "muon_momentum_ns_grouped")
+        return True
 
     def _orthogonalize_classes(self, classes: List[_ShapeClass], eps: float) -> None:
         """U <- NS(U) for every shape class in ONE grouped call (each product of the iteration is one launch over

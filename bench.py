@@ -108,6 +108,8 @@ def main():
                     help="quintic = the reference's production 5-row schedule; simple = constant row with the B split")
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="(debug) fewer layers; the result is then not the metric")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--separate-momentum", action="store_true",
+                    help="(comparison) momentum kernel and Newton-Schulz as separate library calls instead of the fused one")
     ap.add_argument("--seed", type=int, default=1236)
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain device copy run once after the steps (yardstick for HBM byte counters)")
@@ -129,7 +131,7 @@ def main():
     simple = args.coeffs == "simple"
     opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, adjust_lr="spectral_norm",
                use_muonh=True, ns_coefficients=[H.SIMPLE_ROW] * 5 if simple else None,
-               ns_precision="bsplit" if simple else "bf16")
+               ns_precision="bsplit" if simple else "bf16", fuse_momentum=not args.separate_momentum)
 
     for _ in range(args.warmup):  # also warms the momentum so that M != G
         opt.step()

@@ -149,6 +149,29 @@ typedef struct muon_pre_item {
 int muon_momentum(const muon_pre_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
                   float c_mm, float c_mg, float c_um, float c_ug, float l2, void* stream);
 
+/* ---- momentum fused into the Newton-Schulz call ---------------------------------------------------------------
+ * muon_momentum followed by muon_ns_grouped, without the bf16 update U ever being stored in the parameter's
+ * orientation: the momentum kernel writes bf16(U) straight into the (transposed, zero-padded) operand of the iteration
+ * with per-tile sums of squares, and the normalisation 1/(|bf16(U)| + eps) (lit_gpt/optim/muon.py:883-888) is applied by
+ * the first iteration's GEMM epilogues.  Saves one write and two reads of U per step.  Momentum semantics and
+ * coefficients as muon_momentum (muon.py:653-681); a problem is one shape class whose `batch` matrices (rows x cols,
+ * contiguous) are given by HOST arrays of device pointers; `out` receives the result as in muon_ns_problem.
+ * Workspace: muon_ns_grouped_workspace_bytes of the same shapes.  MUON_NS_CAST_INPUT_FIRST is implied, not accepted.
+ */
+typedef struct muon_mns_problem {
+  const void* const* g_ptrs; /* gradients (read; written when l2 != 0) */
+  void* const* m_ptrs;       /* momentum, in place */
+  const void* const* w_ptrs; /* weights, read only when l2 != 0 (may be null otherwise) */
+  void* out;                 /* bf16, [batch][rows][out_ld] */
+  int64_t out_batch_stride;
+  int32_t out_ld;
+  int32_t g_dtype, m_dtype, w_dtype, batch, rows, cols, reserved;
+} muon_mns_problem;
+
+int muon_momentum_ns_grouped(const muon_mns_problem* problems_host, int n_problems, float c_mm, float c_mg, float c_um,
+                             float c_ug, float l2, const float* abc_host, int iters, float eps, int eps_mode,
+                             int prec_mode, int flags, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* ---- multi-tensor weight updates ------------------------------------------------------------
  * x' = x*(1 - lr_wd), or with cautious != 0:  x' = x - lr_wd*x where x*u >= 0  (muon.py:703-718).
  * muon_update_plain:  W <- x' - lr*lr_ratio*U                                   (muon.py:720-722;

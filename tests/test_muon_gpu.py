@@ -165,7 +165,7 @@ def test_hook_state_dict_and_groups(gpu_device):
               dict(params=[lion_vec], algorithm="lion", lr=1e-3)]
     opt = Muon(groups, lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0, newton_schulz_func=hook)
     opt.exclude_from_hyperball(emb)
-    ref = Muon(copy.deepcopy(groups), lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0)
+    ref = Muon(copy.deepcopy(groups), lr=0.02, nesterov=True, use_muonh=True, weight_decay=0.0, fuse_momentum=False)
     for p, q in zip(opt.param_groups[0]["params"], ref.param_groups[0]["params"]):
         g = torch.randn_like(p) * 1e-3
         p.grad, q.grad = g, g.clone()
@@ -341,3 +341,46 @@ def test_step_replays_under_a_hip_graph(gpu_device):
             assert torch.equal(a, b), k
         for a, b in zip(pa, pb):
             assert torch.equal(oa.state[a]["momentum"], ob.state[b]["momentum"])
+
+
+@pytest.mark.parametrize("wdtype,gdtype", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("nesterov", [True, False])
+def test_fused_momentum_equals_separate_calls(gpu_device, wdtype, gdtype, nesterov):
+    """The call that feeds the momentum update straight into the Newton-Schulz operand against momentum kernel + batched
+    Newton-Schulz: momentum buffers bit-identical; weights equal up to the one bf16 rounding of the normalised input that
+    the fused path leaves out (it scales in the first iteration's epilogues instead)."""
+    from archscale_amd.optim.muon import Muon
+    shapes = [(128, 256), (256, 128), (128, 256), (64, 64), (3, 64, 192), (2, 192, 64), (300, 100), (100, 300), (37, 53)]
+    g = torch.Generator().manual_seed(5)
+    W0 = [(torch.randn(*s, generator=g) * 0.02).to(wdtype) for s in shapes]
+    pa = [torch.nn.Parameter(w.clone().to(gpu_device)) for w in W0]
+    pb = [torch.nn.Parameter(w.clone().to(gpu_device)) for w in W0]
+    kw = dict(lr=0.02, mu=0.95, weight_decay=0.01, nesterov=nesterov, use_muonh=True)
+    oa, ob = Muon(pa, fuse_momentum=True, **kw), Muon(pb, fuse_momentum=False, **kw)
+    for step in range(3):
+        grads = [(torch.randn(*s, generator=g) * 1e-3).to(gdtype).to(gpu_device) for s in shapes]
+        for a, b, gr in zip(pa, pb, grads):
+            a.grad, b.grad = gr.clone(), gr.clone()
+        oa.step(); ob.step()
+    assert oa._plans[0][1].fused_probs is not None
+    for a, b, w0 in zip(pa, pb, W0):
+        assert torch.equal(oa.state[a]["momentum"], ob.state[b]["momentum"])
+        assert _rel(a.detach(), b.detach()) < 2e-3
+        if wdtype == torch.float32:
+            assert _rel(a.detach().cpu() - w0, b.detach().cpu() - w0) < 1e-2
+
+
+def test_fused_momentum_falls_back(gpu_device):
+    from archscale_amd.optim.muon import Muon
+    p = torch.nn.Parameter((torch.randn(64, 96) * 0.02).to(gpu_device))
+    p.grad = torch.randn_like(p) * 1e-3
+    opt = Muon([p], lr=0.02, ns_workspace_limit=1)      # nothing fits: separate calls, sliced
+    opt.phase_events = []
+    opt.step()
+    torch.cuda.synchronize()
+    assert [n for n, _, _ in opt.phase_events][:2] == ["momentum", "newton_schulz"]
+    opt2 = Muon([p], lr=0.02)
+    opt2.phase_events = []
+    opt2.step()
+    torch.cuda.synchronize()
+    assert [n for n, _, _ in opt2.phase_events][0] == "momentum+newton_schulz"
