@@ -179,3 +179,55 @@ def test_emerging_host_logic():
     g = o.param_groups[0]
     assert (g["lr"], g["momentum_beta"], g["weight_decay"]) == (3e-4, 0.95, 0.01)
     assert np.isclose(o._extra_scale_factor, 1.0)
+
+
+def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_path):
+    """The K-major GEMM variant issues its LDS transpose reads as inline assembly (the compiler would otherwise wait for
+    every outstanding global->LDS copy before each of them), so the compiler does not know that their results arrive
+    late: the kernel waits explicitly (s_waitcnt lgkmcnt(0)) before the first use. This checks the generated code: no
+    instruction between such a read and the next full LGKM wait may mention the registers the read writes."""
+    import re
+    import subprocess
+    from archscale_amd.build import CSRC, HIPCC_FLAGS, find_hipcc
+    out = tmp_path / "ns_gemm.s"
+    subprocess.run([find_hipcc(), *HIPCC_FLAGS, "--cuda-device-only", "-S", os.path.join(CSRC, "ns_gemm.hip"), "-o", str(out)],
+                   check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    text = out.read_text().splitlines()
+    reg = re.compile(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b")
+
+    def regs(s):
+        found = set()
+        for a, b, c in reg.findall(s):
+            found |= set(range(int(a), int(b) + 1)) if a else {int(c)}
+        return found
+
+    kernels = reads = 0
+    pending, inside, in_asm = set(), False, False
+    for line in text:
+        if "#ASMSTART" in line or "#ASMEND" in line:
+            in_asm = "#ASMSTART" in line
+            continue
+        code = line.split(";")[0].strip()
+        if code.endswith(":") and "ns_gemm_kernel" in code:
+            inside = "ELi3ELb" in code          # MODE_SYRKT instantiations
+            kernels += inside
+            pending = set()
+            continue
+        if not inside or not code or code.startswith("."):
+            continue
+        if code.startswith("s_endpgm"):
+            assert not pending
+            inside = False
+            continue
+        if code.startswith("ds_read_b64_tr_b16") and in_asm:   # the compiler tracks the ones it emits itself
+            dst, addr = code[len("ds_read_b64_tr_b16"):].split(",")[:2]
+            assert not (regs(addr) & pending), line
+            assert not (regs(dst) & pending), line
+            pending |= regs(dst)
+            reads += 1
+            continue
+        if code.startswith("s_waitcnt") and "lgkmcnt(0)" in code:
+            pending = set()
+            continue
+        assert not (regs(code) & pending), f"uses a transpose-read result before the wait: {line}"
+    assert kernels == 2 and reads >= 2 * 12 * 4
