@@ -6,6 +6,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -78,7 +79,7 @@ struct ProfRec {
 };
 std::mutex g_prof_mutex;
 std::vector<ProfRec> g_prof;
-bool g_prof_on = false;
+std::atomic<bool> g_prof_on{false};
 
 hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GroupedGemmParams& g, hipStream_t stream,
                       double flops_algorithmic, double flops_issued) {
@@ -90,8 +91,11 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
   r.flops_issued = flops_issued;
   hipError_t e;
   if ((e = hipEventCreate(&r.start)) != hipSuccess) return e;
-  if ((e = hipEventCreate(&r.stop)) != hipSuccess) return e;
-  if ((e = hipEventRecord(r.start, stream)) != hipSuccess) return e;
+  if ((e = hipEventCreate(&r.stop)) != hipSuccess) { (void)hipEventDestroy(r.start); return e; }
+  if ((e = hipEventRecord(r.start, stream)) != hipSuccess) {
+    (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop);
+    return e;
+  }
   e = launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
   hipError_t e2 = hipEventRecord(r.stop, stream);
   g_prof.push_back(r);
