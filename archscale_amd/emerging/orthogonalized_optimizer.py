@@ -31,19 +31,23 @@ class _Plan:
     """Device tables of one param group: momentum items for every parameter, update items for the batched path."""
 
     def __init__(self, params: List[torch.Tensor], grads: List[torch.Tensor], ratios: Optional[List[float]],
-                 device: torch.device):
+                 device: torch.device, fused: bool = False):
         self.params = params
+        self.device = device
+        self.fused = fused
         chunk = _lib.CHUNK_ELEMS
         n = len(params)
         self.classes: Dict[Tuple[int, ...], List[int]] = {}  # keyed by the full parameter shape
         for i, p in enumerate(params):
             self.classes.setdefault(tuple(p.shape), []).append(i)
-        # U (fp32: the matrix sign normalises in fp32 before rounding) and O (bf16) per shape class
+        # U (fp32: the matrix sign normalises in fp32 before rounding) and O (bf16) per shape class; the fused
+        # momentum + Newton-Schulz call never materialises U
         self.U: Dict[Tuple[int, ...], torch.Tensor] = {}
         self.O: Dict[Tuple[int, ...], torch.Tensor] = {}
         self.slot: List[Tuple[Tuple[int, ...], int]] = [((0, 0), 0)] * n
         for key, idx in self.classes.items():
-            self.U[key] = torch.empty((len(idx), *key), dtype=torch.float32, device=device)
+            if not fused:
+                self.U[key] = torch.empty((len(idx), *key), dtype=torch.float32, device=device)
             self.O[key] = torch.empty((len(idx), *key), dtype=torch.bfloat16, device=device)
             for k, i in enumerate(idx):
                 self.slot[i] = (key, k)
@@ -58,6 +62,17 @@ class _Plan:
         self.post_tab = _DeviceTable(self.post.nbytes, device)
         self.prefix_dev = torch.from_numpy(self.prefix).to(device)
         self.sig: Optional[Tuple] = None
+        self.fused_probs = None
+        self.fused_keep: List = []
+
+    @staticmethod
+    def can_fuse(params: List[torch.Tensor], grads: List[torch.Tensor], bufs: List[torch.Tensor]) -> bool:
+        """One (gradient, buffer, parameter) dtype triple per shape class, as the fused call takes them."""
+        seen: Dict[Tuple[int, ...], Tuple] = {}
+        for p, g, m in zip(params, grads, bufs):
+            if seen.setdefault(tuple(p.shape), (g.dtype, m.dtype, p.dtype)) != (g.dtype, m.dtype, p.dtype):
+                return False
+        return True
 
     def refresh(self, grads: List[torch.Tensor], bufs: List[torch.Tensor]) -> None:
         sig = tuple((p.data_ptr(), g.data_ptr(), m.data_ptr()) for p, g, m in zip(self.params, grads, bufs))
@@ -66,17 +81,38 @@ class _Plan:
         for i, (p, g, m) in enumerate(zip(self.params, grads, bufs)):
             key, k = self.slot[i]
             pre, post = self.pre[i], self.post[i]
-            pre["g"], pre["m"], pre["w"] = g.data_ptr(), m.data_ptr(), p.data_ptr()
-            pre["u"] = self.U[key][k].data_ptr()
-            pre["numel"] = p.numel()
-            pre["g_dtype"], pre["m_dtype"] = _lib.dtype_code(g.dtype), _lib.dtype_code(m.dtype)
-            pre["u_dtype"], pre["w_dtype"] = _lib.DTYPE_F32, _lib.dtype_code(p.dtype)
+            if not self.fused:
+                pre["g"], pre["m"], pre["w"] = g.data_ptr(), m.data_ptr(), p.data_ptr()
+                pre["u"] = self.U[key][k].data_ptr()
+                pre["numel"] = p.numel()
+                pre["g_dtype"], pre["m_dtype"] = _lib.dtype_code(g.dtype), _lib.dtype_code(m.dtype)
+                pre["u_dtype"], pre["w_dtype"] = _lib.DTYPE_F32, _lib.dtype_code(p.dtype)
             post["w"], post["u"] = p.data_ptr(), self.O[key][k].data_ptr()
             post["numel"], post["w_dtype"] = p.numel(), _lib.dtype_code(p.dtype)
             post["lr_ratio"] = self.ratios[i] if self.ratios is not None else 1.0
-        self.pre_tab.upload(self.pre)
+        if not self.fused:
+            self.pre_tab.upload(self.pre)
         self.post_tab.upload(self.post)
         self.sig = sig
+        if self.fused:
+            self._build_fused(grads, bufs)
+
+    def _build_fused(self, grads: List[torch.Tensor], bufs: List[torch.Tensor]) -> None:
+        """muon_mns_problem array: per shape class the (g, m, w) pointers of its matrices in the order of its O buffer."""
+        import ctypes
+        probs = (_lib.MnsProblem * len(self.classes))()
+        keep = []
+        for q, (key, idx) in zip(probs, self.classes.items()):
+            cols = [[t[i].data_ptr() for i in idx] for t in (grads, bufs, self.params)]
+            arrs = [(ctypes.c_void_p * len(idx))(*c) for c in cols]
+            keep.append(arrs)
+            q.g_ptrs, q.m_ptrs, q.w_ptrs = (ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p)) for a in arrs)
+            q.out, q.out_batch_stride, q.out_ld = self.O[key].data_ptr(), key[0] * key[1], key[1]
+            i0 = idx[0]
+            q.g_dtype, q.m_dtype = _lib.dtype_code(grads[i0].dtype), _lib.dtype_code(bufs[i0].dtype)
+            q.w_dtype = _lib.dtype_code(self.params[i0].dtype)
+            q.batch, q.rows, q.cols = len(idx), key[0], key[1]
+        self.fused_probs, self.fused_keep = probs, keep
 
 
 class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
@@ -115,6 +151,9 @@ class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
         self.per_module_grad_rms: Dict[str, float] = {}
         super().__init__(params, dict(lr=lr, momentum_beta=momentum_beta, weight_decay=weight_decay, **kwargs))
         self.scaled_orthogonalize_fn = scaled_orthogonalize_fn
+        #: batched path only: momentum and Newton-Schulz in one library call that never stores the blended
+        #: momentum (its bf16 rounding goes straight into the operand of the iteration)
+        self.fuse_momentum = True
         self._plans: Dict[int, Tuple[Tuple, _Plan]] = {}
 
     # A subclass whose update is "Newton-Schulz with a coefficient table, times a per-shape scale" returns
@@ -164,12 +203,13 @@ class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
         batched = (recipe is not None and self._uses_default_orthogonalize() and not logging_on
                    and all(t.ndim == 2 for t in local))
         ratios = [recipe[4](t.shape[-2], t.shape[-1]) for t in local] if batched else None
+        fused = batched and self.fuse_momentum and _Plan.can_fuse(local, grads, bufs)
 
         sig = (tuple((id(p), tuple(t.shape), t.dtype, g.dtype) for p, t, g in zip(params, local, grads)), batched,
-               tuple(ratios) if ratios else None)
+               tuple(ratios) if ratios else None, fused)
         cached = self._plans.get(gi)
         if cached is None or cached[0] != sig:
-            plan = _Plan(local, grads, ratios, device)
+            plan = _Plan(local, grads, ratios, device, fused)
             self._plans[gi] = (sig, plan)
         else:
             plan = cached[1]
@@ -181,6 +221,19 @@ class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
             stream = _lib.current_stream_ptr(device)
             # grad (+= wd*p for l2);  buf <- lerp(buf, grad, 1-beta);  U = lerp(grad, buf, beta) | buf
             um, ug = (beta, 1.0 - beta) if self.use_nesterov else (1.0, 0.0)
+            if fused:
+                coeffs, eps, eps_mode, prec, _ = recipe
+                pm = _lib.PREC_BF16_BSPLIT if prec == "bsplit" else _lib.PREC_BF16
+                em = _lib.EPS_CLAMP if eps_mode == "clamp" else _lib.EPS_ADD
+                need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in plan.fused_probs)
+                ws = _lib.workspace(device, need)
+                _lib.check(L.muon_momentum_ns_grouped(plan.fused_probs, len(plan.fused_probs), beta, 1.0 - beta, um, ug, l2,
+                                                      _lib.abc_array(coeffs), len(coeffs), eps, em, pm,
+                                                      _lib.ns_bsplit_tail(ns.BSPLIT_TAIL), ws.data_ptr(), ws.numel(),
+                                                      stream), "muon_momentum_ns_grouped")
+                _lib.check(L.muon_update_plain(plan.post_tab.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(local),
+                                               plan.chunks, lr, lr_wd, 0, stream), "muon_update_plain")
+                return
             _lib.check(L.muon_momentum(plan.pre_tab.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(local),
                                        plan.chunks, beta, 1.0 - beta, um, ug, l2, stream), "muon_momentum")
             if batched:

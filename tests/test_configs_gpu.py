@@ -191,3 +191,78 @@ def test_config2_muon_ball_full_step(gpu_device):
     ev1.record()
     torch.cuda.synchronize()
     print(f"config 2 MuonBall: {ev0.elapsed_time(ev1) / 3:.1f} ms/step (50 power-iteration rounds, msign 5 steps)", flush=True)
+
+
+def test_config2_emerging_muon_full_step(gpu_device):
+    """emerging_optimizers-style Muon (EMA momentum, polar-express msign, decoupled weight decay) over the depth-16
+    dense parameter set in fp32 (msign takes fp32 only, spectral_ball_utils.py:25-74); sampled matrices against the CPU
+    oracle, then the step time."""
+    from archscale_amd.emerging import Muon as EMuon
+    from oracle import muon_oracle as O
+    layer = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (5632, 2048), (5632, 2048), (2048, 5632)]
+    g = torch.Generator(device=gpu_device).manual_seed(1242)
+    params, grads = [], []
+    for _ in range(16):
+        for s in layer:
+            params.append(torch.nn.Parameter(torch.randn(*s, generator=g, device=gpu_device) * 0.02))
+            grads.append(torch.randn(*s, generator=g, device=gpu_device) * 1e-3)
+    for p, gr in zip(params, grads):
+        p.grad = gr
+    lr, beta, wd = 0.02, 0.95, 0.01
+    opt = EMuon(params, lr=lr, momentum_beta=beta, weight_decay=wd, use_nesterov=True, num_ns_steps=5,
+                scale_mode="spectral_mup")
+    sample = [0, 1, 4, 6, 111]
+    w0 = {i: params[i].detach().cpu().clone() for i in sample}
+    opt.step()
+    torch.cuda.synchronize()
+    for i in sample:
+        x, m = w0[i].clone(), torch.zeros_like(w0[i])
+        O.emerging_muon_step(x, grads[i].cpu().clone(), m, lr=lr, beta=beta, wd=wd, nesterov=True, wd_method="decoupled",
+                             steps=5, scale_mode="spectral_mup", extra_scale=1.0, ns_storage="fp32")
+        assert _rel(params[i].detach(), x) <= W_TOL
+        d_got, d_want = params[i].detach().float().cpu() - w0[i].float(), x.float() - w0[i].float()
+        assert _rel(d_got, d_want) <= 2e-2         # fp32 weights: the delta carries the Newton-Schulz error only
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(3):
+        opt.step()
+    ev1.record()
+    torch.cuda.synchronize()
+    print(f"config 2 emerging Muon: {ev0.elapsed_time(ev1) / 3:.1f} ms/step (msign 5 steps, hi+lo split on the last 3)", flush=True)
+
+
+def test_scalar_groups_throughput(gpu_device):
+    """AdamW, hyperball-AdamW and Lion over the non-matrix tensors of the depth-16 model (token embedding and
+    lm_head 50304 x 2048, 33 norm vectors), bf16 state: one multi-tensor launch each; prints the HBM rate against the
+    bytes each algorithm has to move and checks it against a loose floor."""
+    from archscale_amd.optim import scalar_opts as H
+    dev = gpu_device
+    g = torch.Generator(device=dev).manual_seed(5)
+    shapes = [(50304, 2048), (50304, 2048)] + [(2048,)] * 33
+    mk = lambda scale: [(torch.randn(*s, generator=g, device=dev) * scale).to(torch.bfloat16) for s in shapes]
+    X, G, M = mk(0.02), mk(1e-3), mk(1e-3)
+    V = [(torch.rand(*s, generator=g, device=dev) * 1e-6).to(torch.bfloat16) for s in shapes]
+    n = sum(x.numel() for x in X)
+    # bytes per element with bf16 everywhere: AdamW reads w,g,m,v and writes w,m,v; Lion reads w,g,m and writes w,m;
+    # hyperball: pass 1 reads w,g,m,v and writes m,v, pass 2 reads w,m,v and writes w (2-D tensors only)
+    cases = [
+        ("adamw", 14, lambda step: H.adamw_update_foreach(X, G, M, V, 1e-3, 0.9, 0.95, 0.1, step, 1e-8, False)),
+        ("lion", 10, lambda step: H.lion_update_foreach(X, G, M, 1e-4, 0.9, 0.99, 0.1, False)),
+        ("hyperball", 20, lambda step: H.hyperball_adamw_update_foreach(X[:2], G[:2], M[:2], V[:2], 1e-3, 0.9, 0.95, 0.1,
+                                                                       step, 1e-8, False)),
+    ]
+    for name, bpe, fn in cases:
+        elems = n if name != "hyperball" else X[0].numel() * 2
+        fn(1)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for s in range(5):
+            fn(2 + s)
+        ev1.record()
+        torch.cuda.synchronize()
+        ms = ev0.elapsed_time(ev1) / 5
+        rate = elems * bpe / (ms * 1e-3) / 1e12
+        print(f"scalar groups {name}: {elems / 1e6:.0f} M elements, {ms:.3f} ms/step, {rate:.2f} TB/s of {bpe} B/elem", flush=True)
+        assert all(torch.isfinite(x.float()).all() for x in X[:1])
+        assert rate > 2.0
