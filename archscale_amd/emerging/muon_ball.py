@@ -12,7 +12,8 @@ sigma, an in-place retraction, msign of the momentum and the update.  Here a par
   1 multi-tensor launch   W <- f * decay * W - lr * scale * Phi  with the retraction factor f taken from sigma on the
                           device.
 
-Pieces are described once per parameter set (``_Piece``) and cached.
+When no parameter is split (every piece is a whole matrix) the momentum launch and the msign call are ONE library call
+that never stores the blended momentum.  Pieces are described once per parameter set (``_Piece``) and cached.
 """
 from __future__ import annotations
 
@@ -140,6 +141,8 @@ class _BallPlan:
             q.dtype, q.ld, q.batch, q.rows, q.cols = _lib.dtype_code(dt), ld, len(idx), rows, cols
             q.flags = _lib.SN_TRANSPOSED if transposed else 0
         for q, (gkey, idx) in zip(self.ns_probs, self.ns_groups):
+            if base.fused:
+                break   # every piece is a whole matrix: the base plan's fused momentum + msign problems cover them
             pc = self.pieces[idx[0]]
             if gkey[0] == "tmp":
                 i = idx[0]
@@ -336,12 +339,17 @@ class MuonBall(OrthogonalizedOptimizer):
         wd = group.get("wd_mult", 1.0) * group["weight_decay"]
         lr_wd, l2 = weight_decay_terms(self.weight_decay_method, lr, wd)
 
-        sig = tuple((id(p), tuple(t.shape), t.dtype, g.dtype, getattr(p, "param_name", None),
-                     getattr(p, "num_local_experts", None), getattr(p, "is_gated", None))
-                    for p, t, g in zip(params, local, grads))
+        sig = (tuple((id(p), tuple(t.shape), t.dtype, g.dtype, getattr(p, "param_name", None),
+                      getattr(p, "num_local_experts", None), getattr(p, "is_gated", None))
+                     for p, t, g in zip(params, local, grads)), self.fuse_momentum, self.log_per_module_grad_rms)
         cached = self._ball_plans.get(gi)
         if cached is None or cached[0] != sig:
-            base = _Plan(local, grads, None, device)
+            # momentum fused into the msign call when every piece is a whole, contiguous matrix
+            whole = all(pc.gather is None and pc.off == 0 and pc.ld == pc.cols and pc.rows * pc.cols == t.numel()
+                        for i, (p, t) in enumerate(zip(params, local)) for pc in self._pieces_of(i, p, t))
+            fused = (self.fuse_momentum and whole and not self.log_per_module_grad_rms
+                     and _Plan.can_fuse(local, grads, bufs))
+            base = _Plan(local, grads, None, device, fused)
             plan = _BallPlan(self, base, params, local, device)
             self._ball_plans[gi] = (sig, plan)
         else:
@@ -356,8 +364,9 @@ class MuonBall(OrthogonalizedOptimizer):
             stream = _lib.current_stream_ptr(device)
             # grad (+= wd*p for l2);  buf <- lerp(buf, grad, 1-beta);  U = lerp(grad, buf, beta) | buf   (fp32)
             um, ug = (beta, 1.0 - beta) if self.use_nesterov else (1.0, 0.0)
-            _lib.check(L.muon_momentum(base.pre_tab.dev.data_ptr(), base.prefix_dev.data_ptr(), len(local), base.chunks,
-                                       beta, 1.0 - beta, um, ug, l2, stream), "muon_momentum")
+            if not base.fused:
+                _lib.check(L.muon_momentum(base.pre_tab.dev.data_ptr(), base.prefix_dev.data_ptr(), len(local),
+                                           base.chunks, beta, 1.0 - beta, um, ug, l2, stream), "muon_momentum")
             if self.log_per_module_grad_rms:
                 for p, i in zip(params, range(len(params))):
                     name = getattr(p, "param_name", None)
@@ -384,11 +393,19 @@ class MuonBall(OrthogonalizedOptimizer):
             # Phi = msign(U) for every piece, written into the bf16 update buffers
             n_ns = len(plan.ns_groups)
             pm = _lib.PREC_BF16_BSPLIT
-            ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(plan.ns_probs, n_ns, pm))
             coeffs = msign_schedule(self.msign_steps)
-            _lib.check(L.muon_ns_grouped(plan.ns_probs, n_ns, _lib.abc_array(coeffs), len(coeffs), 1e-7, _lib.EPS_CLAMP,
-                                         pm, _lib.ns_bsplit_tail(ns.BSPLIT_TAIL), ws.data_ptr(), ws.numel(), stream),
-                       "muon_ns_grouped")
+            if base.fused:
+                need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in base.fused_probs)
+                ws = _lib.workspace(device, need)
+                _lib.check(L.muon_momentum_ns_grouped(base.fused_probs, len(base.fused_probs), beta, 1.0 - beta, um, ug, l2,
+                                                      _lib.abc_array(coeffs), len(coeffs), 1e-7, _lib.EPS_CLAMP, pm,
+                                                      _lib.ns_bsplit_tail(ns.BSPLIT_TAIL), ws.data_ptr(), ws.numel(),
+                                                      stream), "muon_momentum_ns_grouped")
+            else:
+                ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(plan.ns_probs, n_ns, pm))
+                _lib.check(L.muon_ns_grouped(plan.ns_probs, n_ns, _lib.abc_array(coeffs), len(coeffs), 1e-7,
+                                             _lib.EPS_CLAMP, pm, _lib.ns_bsplit_tail(ns.BSPLIT_TAIL), ws.data_ptr(),
+                                             ws.numel(), stream), "muon_ns_grouped")
             for i, pc in enumerate(plan.pieces):
                 if pc.gather is None:
                     continue

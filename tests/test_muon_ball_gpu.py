@@ -313,3 +313,32 @@ def test_spectral_norm_of_the_transpose(gpu_device):
         assert abs(want_t - want) / want > 2 * SIGMA_TOL          # the two orientations really differ here
     q.flags = 2
     assert L.muon_spectral_norm(prob, 1, 4, ws.data_ptr(), ws.numel(), 0) < 0
+
+
+def test_fused_momentum_matches_separate_calls(gpu_device):
+    """Unsplit parameters take the fused momentum + msign call; same buffers and (up to where the update is rounded to
+    bf16) the same weights as the separate momentum launch."""
+    from archscale_amd.emerging import MuonBall
+    shapes = [(256, 512), (512, 256), (256, 512), (192, 320)]
+    outs = []
+    for fuse in (True, False):
+        g = torch.Generator().manual_seed(77)
+        params = [torch.nn.Parameter((torch.randn(*s, generator=g) * 0.05).to(gpu_device)) for s in shapes]
+        opt = MuonBall(params, lr=0.02, momentum_beta=0.9, weight_decay=0.1, use_nesterov=True, weight_decay_method="l2",
+                       power_iteration_steps=20, msign_steps=5)
+        opt.fuse_momentum = fuse
+        w0 = [p.detach().clone() for p in params]
+        for k in range(2):
+            gg = torch.Generator().manual_seed(90 + k)
+            for p, s in zip(params, shapes):
+                p.grad = (torch.randn(*s, generator=gg) * 1e-2).to(gpu_device)
+            opt.step()
+        torch.cuda.synchronize()
+        plan = next(iter(opt._ball_plans.values()))[1]
+        assert plan.base.fused == fuse
+        outs.append(([p.detach().clone() for p in params], [opt.state[p]["momentum_buffer"].clone() for p in params], w0))
+    (wf, mf, w0), (ws, ms, _) = outs
+    rel = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
+    for a, b, m1, m2, w in zip(wf, ws, mf, ms, w0):
+        assert rel(m1, m2) <= 2e-3
+        assert rel(a - w, b - w) <= 1e-2
