@@ -44,11 +44,11 @@ int pick_tile(int m, int n) {
   return cost(256, 1.0) <= cost(128, 1.25) ? 256 : 128;
 }
 
-NsPlan make_plan(int batch, int rows, int cols, int prec_mode) {
+NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   NsPlan p;
   p.m = rows < cols ? rows : cols;
   p.n = rows < cols ? cols : rows;
-  p.tile = pick_tile(p.m, p.n);
+  p.tile = tile ? tile : pick_tile(p.m, p.n);
   p.Mp = (int)round_up(p.m, p.tile);
   p.Np = (int)round_up(p.n, p.tile);
   p.cpm = (int)(((long)rows * cols + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
@@ -69,6 +69,26 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode) {
 }
 
 inline long sym_tiles(int t) { return (long)t * (t + 1) / 2; }
+
+// workspace bound of one problem: the larger of the two tile configurations (a call with few tiles in total takes the
+// small one, see ns_grouped_impl)
+size_t plan_bytes_bound(int batch, int rows, int cols, int prec_mode) {
+  if (getenv("ARCHSCALE_MUON_TILE")) return make_plan(batch, rows, cols, prec_mode).total;
+  return std::max(make_plan(batch, rows, cols, prec_mode, 256).total, make_plan(batch, rows, cols, prec_mode, 128).total);
+}
+
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
 
 // Optional per-launch timing of the Newton-Schulz GEMMs (muon_profile_begin / muon_profile_collect):
 // one pair of HIP events around every GEMM launch, on the stream the kernel runs on.
@@ -119,7 +139,7 @@ const char* muon_status_string(int status) {
 
 size_t muon_ns_workspace_bytes(int batch, int rows, int cols, int prec_mode) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
-  return make_plan(batch, rows, cols, prec_mode).total;
+  return plan_bytes_bound(batch, rows, cols, prec_mode);
 }
 
 void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode, double* dense, double* symmetric,
@@ -161,7 +181,7 @@ size_t muon_ns_grouped_workspace_bytes(const muon_ns_problem* problems_host, int
   for (int i = 0; i < n_problems; ++i) {
     const muon_ns_problem& q = problems_host[i];
     if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return 0;
-    total += make_plan(q.batch, q.rows, q.cols, prec_mode).total;
+    total += plan_bytes_bound(q.batch, q.rows, q.cols, prec_mode);
   }
   return total;
 }
@@ -186,12 +206,22 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
 
   std::vector<NsProblem> pr(n_problems);
   size_t off = 0;
+  // A call whose smallest launch (the symmetric products) would not even occupy half of the compute units with 256x256
+  // tiles takes the 128x128 configuration for every problem: four times the blocks, a quarter of the time per block.
+  long sym_blocks = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    const muon_ns_problem& q = problems_host[i];
+    if (q.batch <= 0 || q.rows <= 0 || q.cols <= 0) return MUON_E_ARG;
+    const NsPlan pl = make_plan(q.batch, q.rows, q.cols, prec_mode);
+    sym_blocks += (long)q.batch * sym_tiles(pl.Mp / pl.tile);
+  }
+  const int force_tile = (!getenv("ARCHSCALE_MUON_TILE") && sym_blocks * 2 < compute_units()) ? 128 : 0;
   for (int i = 0; i < n_problems; ++i) {
     NsProblem& P = pr[i];
     P.q = problems_host[i];
     const int st = check_problem(P.q, fused != nullptr);
     if (st) return st;
-    P.pl = make_plan(P.q.batch, P.q.rows, P.q.cols, prec_mode);
+    P.pl = make_plan(P.q.batch, P.q.rows, P.q.cols, prec_mode, force_tile);
     // byte offsets inside one matrix are 32-bit in the GEMM loader
     if ((double)P.pl.Mp * P.pl.Np * 2.0 >= 4294967296.0) return MUON_E_UNSUPPORTED;
     if (off + P.pl.total > ws_bytes) return MUON_E_WORKSPACE;
