@@ -431,7 +431,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
         }
       }
 
-    auto store_wave = [&](__bf16* Cdst) {
+    auto store_wave = [&](__bf16* Cdst, int lane) {
+      const int l32 = lane & 31, hi = lane >> 5;
       // W[c][r] <- bf16(acc)
 #pragma unroll
       for (int i = 0; i < FM; ++i)
@@ -505,7 +506,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
       }
     };
 
-    store_wave(p.C);
+    store_wave(p.C, lane);
     if (SPLIT && MODE == MODE_SYRK2) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -515,7 +516,11 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[i][j][e] -= bf16_to_f32(bf16_bits(acc[i][j][e]));
       __builtin_amdgcn_sched_barrier(0);
-      store_wave(p.C2);
+      // the second copy of the store code gets its lane id through an opaque move, so that its addresses are computed
+      // here and not hoisted above the first copy (where they cost hundreds of spilled registers)
+      int lane2 = lane;
+      asm volatile("" : "+v"(lane2));
+      store_wave(p.C2, lane2);
     }
     return;
   }
@@ -570,7 +575,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   if (!SYRK_PLAIN) __syncthreads();  // the addend image is consumed; LDS is free again
 
   // stores the accumulators as bf16 to Cdst (row-major image) and to its transposed / mirrored image
-  auto store_all = [&](__bf16* Cdst) {
+  auto store_all = [&](__bf16* Cdst, int lane) {
+    const int l32 = lane & 31, hi = lane >> 5;
     // 2. transposed image
     const bool want_t = SYM ? !diag : (p.Ct != nullptr);
     if (want_t) {
@@ -619,7 +625,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     }
   };
 
-  store_all(p.C);
+  store_all(p.C, lane);
   if (SPLIT && MODE == MODE_SYRK2) {
     __builtin_amdgcn_sched_barrier(0);
     // low half of the bf16 split: acc <- acc - bf16(acc), stored the same way to C2
@@ -631,7 +637,9 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
         for (int e = 0; e < 16; ++e) acc[i][j][e] -= bf16_to_f32(bf16_bits(acc[i][j][e]));
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
-    store_all(p.C2);
+    int lane2 = lane;
+    asm volatile("" : "+v"(lane2));   // as above: keep the second copy's addresses out of the first copy
+    store_all(p.C2, lane2);
   }
 }
 
