@@ -22,6 +22,7 @@ ALGO_ADAMW, ALGO_LION = 0, 1
 RETRACT_HARD, RETRACT_DYNAMIC = 0, 1
 SN_TRANSPOSED = 1
 NS_CAST_INPUT_FIRST = 1
+NS_NO_NORMALIZE = 2
 CHUNK_ELEMS = 8192
 ABI_VERSION = 2
 

@@ -200,7 +200,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   const bool split_any = prec_mode == MUON_PREC_BF16_BSPLIT;
   const int split_tail = (flags >> 8) & 0xff;   // 0: every iteration keeps B as a hi+lo pair; t: only the last t
-  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | 0xff00)) return MUON_E_ARG;
+  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | MUON_NS_NO_NORMALIZE | 0xff00)) return MUON_E_ARG;
+  const bool normalize = !(flags & MUON_NS_NO_NORMALIZE);
+  if (!normalize && fused) return MUON_E_ARG;
   bool split = split_any;
   const int cast_first = (flags & MUON_NS_CAST_INPUT_FIRST) ? 1 : 0;
 
@@ -249,15 +251,18 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const NsProblem& P = pr[i];
     const NsPlan& pl = P.pl;
     const long xs = (long)pl.Mp * pl.Np;
-    e = launch_norm_scale(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                          P.q.cols, eps, eps_mode, P.partial, P.scale, stream);
-    if (e != hipSuccess) return (int)e;
+    const float* sc = normalize ? P.scale : nullptr;   // null: copy unscaled
+    if (normalize) {
+      e = launch_norm_scale(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
+                            P.q.cols, eps, eps_mode, P.partial, P.scale, stream);
+      if (e != hipSuccess) return (int)e;
+    }
     if (!P.tall)
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, P.scale, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
+                        P.q.cols, sc, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
     else
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, P.scale, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream);
+                        P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream);
     if (e != hipSuccess) return (int)e;
   }
   // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials

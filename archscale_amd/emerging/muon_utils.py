@@ -5,7 +5,7 @@ import torch
 
 from ..optim import newton_schulz_hip as ns
 
-__all__ = ["newton_schulz"]
+__all__ = ["newton_schulz", "newton_schulz_step_tsyrk"]
 
 _COEFFICIENT_SETS = {
     "simple": [(3.4445, -4.7750, 2.0315)],
@@ -63,3 +63,15 @@ def newton_schulz(x: torch.Tensor, steps: int, coefficient_type: str = "polar_ex
     out = ns.newton_schulz(x, rows, eps, eps_mode="clamp", prec="bsplit", cast_input_first=False,
                            bsplit_tail=ns.BSPLIT_TAIL)
     return out.to(torch.float32)
+
+
+def newton_schulz_step_tsyrk(X: torch.Tensor, a: float, b: float, c: float, tp_group=None) -> torch.Tensor:
+    """One iteration ``aX + (bA + cA^2)X, A = XX^T`` on a bf16 matrix as it is, no normalisation
+    (emerging_optimizers/orthogonalized_optimizers/muon_utils.py:262-287). Returns a new bf16 tensor."""
+    if X.dtype != torch.bfloat16:
+        raise ValueError(f"X must be bfloat16, got {X.dtype}")
+    if X.ndim != 2:
+        raise ValueError("X must be a 2-D matrix")
+    if tp_group is not None:
+        raise NotImplementedError("this build runs Newton-Schulz on one GPU; tp_group must be None")
+    return ns.newton_schulz(X, [(float(a), float(b), float(c))], 0.0, prec="bsplit", normalize=False)

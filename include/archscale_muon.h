@@ -37,6 +37,9 @@ extern "C" {
 /* flags of muon_ns_batched */
 #define MUON_NS_CAST_INPUT_FIRST 1 /* fp32 input: round to bf16 BEFORE taking the norm (muon.py:883-888); default is
                                       normalise in fp32, then round (spectral_ball_utils.py:46-54) */
+#define MUON_NS_NO_NORMALIZE 2     /* iterate on the input as it is (no Frobenius normalisation; eps is ignored): one call
+                                      with iters = 1 is newton_schulz_step_tsyrk
+                                      (emerging_optimizers/orthogonalized_optimizers/muon_utils.py:262-287) */
 #define MUON_NS_BSPLIT_TAIL(t) (((t) & 0xff) << 8) /* with MUON_PREC_BF16_BSPLIT: only the last t iterations keep B as a
                                                       hi+lo pair (0 = all); the rounding of B in the last iterations
                                                       dominates the error of the result */

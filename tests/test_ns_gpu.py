@@ -195,3 +195,21 @@ def test_bsplit_tail(gpu_device):
     st = _lib.lib().muon_ns_batched(Gd.data_ptr(), 0, 384 * 1024, 1024, full.data_ptr(), 384 * 1024, 1024, 3, 384, 1024, abc, 5,
                                     1e-7, 0, 1, 1 << 20, ws.data_ptr(), ws.numel(), 0)
     assert st < 0
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (384, 200), (100, 36)])
+def test_single_step_without_normalisation(gpu_device, shape):
+    """newton_schulz_step_tsyrk: one iteration on the matrix as it is (wide and tall inputs; the tall one is iterated
+    transposed inside, which is the same polynomial)."""
+    from archscale_amd.emerging.muon_utils import newton_schulz_step_tsyrk
+    a, b, c = 3.4445, -4.7750, 2.0315
+    X = (_randn(shape, 5).float() / max(shape) ** 0.5 * 0.6).to(torch.bfloat16)   # singular values below ~1.2
+    got = newton_schulz_step_tsyrk(X.to(gpu_device), a, b, c)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and got.shape == X.shape
+    Xd = X.double()
+    A = Xd @ Xd.T
+    want = a * Xd + (b * A + c * A @ A) @ Xd
+    assert _rel(got, want) <= 4e-3          # one bf16 rounding of A, of B (hi+lo) and of the result
+    with pytest.raises(ValueError):
+        newton_schulz_step_tsyrk(X.float().to(gpu_device), a, b, c)
