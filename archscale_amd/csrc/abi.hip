@@ -122,6 +122,46 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
   return e != hipSuccess ? e : e2;
 }
 
+// One product over all problems of a 256-tile launch.  When the last round of the grid would hold only a few tiles, the
+// full rounds run as they are and the tiles of the last round are handed, as four 128x128 quadrants each, to the small
+// configuration: a quarter of the time per block instead of a whole round for a few tiles.  The small configuration
+// runs at about half the rate of the large one, so this pays for at most QUARTER_MAX_TAIL tiles (measured: a tail of
+// 160 tiles on the depth-16 set costs 83 us quartered against 57 us as it is; tails of 16 and 128 tiles of single
+// 8192x8192 and 4096x14336 matrices: 10.33 -> 9.80 ms and 4.58 -> 4.44 ms per call); a launch smaller than one round
+// is quartered as a whole up to QUARTER_MAX_ALONE tiles.  ARCHSCALE_MUON_QUARTER=0 switches it off.
+constexpr int QUARTER_MAX_TAIL = 128, QUARTER_MAX_ALONE = 176;
+hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp, hipStream_t stream,
+                         double fa, double fi) {
+  static const bool enabled = !(getenv("ARCHSCALE_MUON_QUARTER") && atoi(getenv("ARCHSCALE_MUON_QUARTER")) == 0);
+  const int total = gp.tile_start[gp.n_groups];
+  const int round = 256;
+  const int full = total / round * round, tail = total - full;
+  if (!enabled || tile != 256 || tail == 0 || tail > (full > 0 ? QUARTER_MAX_TAIL : QUARTER_MAX_ALONE))
+    return timed_gemm(tile, mode, split, final_, gp, stream, fa, fi);
+  const double share = (double)full / total;
+  if (full > 0) {
+    GroupedGemmParams m = gp;
+    for (int i = 0; i <= gp.n_groups; ++i) m.tile_start[i] = std::min(gp.tile_start[i], full);
+    hipError_t e = timed_gemm(tile, mode, split, final_, m, stream, fa * share, fi * share);
+    if (e != hipSuccess) return e;
+  }
+  GroupedGemmParams q = {};
+  q.quarter = 1;
+  for (int i = 0; i < gp.n_groups; ++i) {
+    const int s = gp.tile_start[i], e = gp.tile_start[i + 1];
+    const int f = std::max(s, full);
+    if (e <= f) continue;
+    GemmParams g = gp.g[i];
+    g.tilesM *= 2;
+    g.tilesN *= 2;
+    g.qt_first = f - s;
+    q.g[q.n_groups] = g;
+    q.tile_start[q.n_groups + 1] = q.tile_start[q.n_groups] + 4 * (e - f);
+    ++q.n_groups;
+  }
+  return timed_gemm(128, mode, split, final_, q, stream, fa * (1.0 - share), fi * (1.0 - share));
+}
+
 }  // namespace
 
 extern "C" {
@@ -302,7 +342,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       double fa = 0.0, fi = 0.0;
       auto flush = [&]() -> hipError_t {
         if (gp.n_groups == 0) return hipSuccess;
-        hipError_t err = timed_gemm(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi);
+        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi);
         gp = GroupedGemmParams{};
         fa = fi = 0.0;
         return err;

@@ -31,14 +31,19 @@ struct GemmParams {
   float alpha, beta;
   const float* scale;    // per batch element, or null: SYRK / SYRKT multiply the product by scale^2, BX the result by scale
   int m_valid, n_valid;  // true extents for the bounds-checked final store
+  int qt_first;          // quarter mode: first tile of this problem (in its own 2x coarser enumeration) that is covered
 };
 
 // Several independent problems of one kind (same tile configuration, mode, split and final flags) in ONE
 // launch: block b works on problem g with tile_start[g] <= b < tile_start[g+1].  Passed by value as a
 // kernel argument (about 1.3 KiB).
 constexpr int MAX_GROUPS = 8;
+// Quarter mode: the blocks of the launch are the four half-size tiles of each tile of a 2x coarser enumeration
+// (tilesM, tilesN count the fine tiles; block 4q + s is quadrant s of coarse tile qt_first + q).  It lets the 128x128
+// configuration finish the last, partly filled round of a 256x256 launch.
 struct GroupedGemmParams {
   int n_groups;
+  int quarter;
   int tile_start[MAX_GROUPS + 1];
   GemmParams g[MAX_GROUPS];
 };

@@ -89,19 +89,32 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   int grp = 0;
   while (grp + 1 < gp.n_groups && logical >= gp.tile_start[grp + 1]) ++grp;
   const GemmParams p = gp.g[grp];
-  const int local = logical - gp.tile_start[grp];
-  const int tiles_per_mat = SYM ? (p.tilesM * (p.tilesM + 1)) / 2 : p.tilesM * p.tilesN;
+  int local = logical - gp.tile_start[grp];
+  // grid the tile index is decoded in: the problem's own, or the 2x coarser one whose tiles this launch quarters
+  int dM = p.tilesM, dN = p.tilesN, quadrant = 0;
+  if (gp.quarter) {
+    quadrant = local & 3;
+    local = p.qt_first + (local >> 2);
+    dM >>= 1;
+    dN >>= 1;
+  }
+  const int tiles_per_mat = SYM ? (dM * (dM + 1)) / 2 : dM * dN;
   const int b = local / tiles_per_mat;
   int t = local - b * tiles_per_mat;
   int ti, tj;
   if (SYM) {
     ti = 0;
-    int rowlen = p.tilesM;
+    int rowlen = dM;
     while (t >= rowlen) { t -= rowlen; ++ti; --rowlen; }
     tj = ti + t;
   } else {
-    tj = t / p.tilesM;
-    ti = t - tj * p.tilesM;
+    tj = t / dM;
+    ti = t - tj * dM;
+  }
+  if (gp.quarter) {
+    ti = 2 * ti + (quadrant >> 1);
+    tj = 2 * tj + (quadrant & 1);
+    if (SYM && ti > tj) return;   // lower quadrant of a diagonal tile: its mirror image covers it
   }
   const int R0 = ti * BM, C0 = tj * BN;
 
@@ -697,8 +710,21 @@ static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGem
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
                                   hipStream_t stream) {
   if (gp.n_groups < 1 || gp.n_groups > MAX_GROUPS) return hipErrorInvalidValue;
-  for (int i = 0; i < gp.n_groups; ++i)
-    if (gp.g[i].K % BK != 0 || gp.g[i].K <= 0 || gp.tile_start[i + 1] < gp.tile_start[i]) return hipErrorInvalidValue;
+  const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2 || mode == MODE_SYRKT);
+  for (int i = 0; i < gp.n_groups; ++i) {
+    const GemmParams& g = gp.g[i];
+    if (g.K % BK != 0 || g.K <= 0 || gp.tile_start[i + 1] < gp.tile_start[i]) return hipErrorInvalidValue;
+    // every block must decode to a tile inside the problem
+    const long blocks = (long)gp.tile_start[i + 1] - gp.tile_start[i];
+    if (!gp.quarter) {
+      if (blocks > ns_gemm_tiles(mode, g)) return hipErrorInvalidValue;
+    } else {
+      if ((g.tilesM & 1) || (!sym && (g.tilesN & 1)) || g.qt_first < 0 || (blocks & 3)) return hipErrorInvalidValue;
+      const long cm = g.tilesM / 2, cn = g.tilesN / 2;
+      const long coarse = (long)g.batch * (sym ? cm * (cm + 1) / 2 : cm * cn);
+      if (g.qt_first + blocks / 4 > coarse) return hipErrorInvalidValue;
+    }
+  }
   if (tile == 256) return launch_cfg<256, 256, 128, 64>(mode, split, final_, gp, stream);
   if (tile == 128) return launch_cfg<128, 128, 64, 64>(mode, split, final_, gp, stream);
   return hipErrorInvalidValue;

@@ -213,3 +213,19 @@ def test_single_step_without_normalisation(gpu_device, shape):
     assert _rel(got, want) <= 4e-3          # one bf16 rounding of A, of B (hi+lo) and of the result
     with pytest.raises(ValueError):
         newton_schulz_step_tsyrk(X.float().to(gpu_device), a, b, c)
+
+
+def test_quartered_tail_matches_other_grids(ns, gpu_device):
+    """A launch whose last round holds few tiles hands them to the 128x128 configuration as quadrants. Which tiles
+    those are depends on the batch, the arithmetic of a tile does not: the same matrix gives the same bits alone
+    (small-call path), in a batch of 8 (tail of 32 tiles) and in a batch of 16 (tail of 64 tiles)."""
+    G = _randn((16, 2048, 2048), 91).to(gpu_device)
+    all16 = ns.newton_schulz(G)
+    first8 = ns.newton_schulz(G[:8])
+    alone = ns.newton_schulz(G[3])
+    torch.cuda.synchronize()
+    assert torch.equal(all16[:8], first8)
+    assert torch.equal(all16[3], alone)
+    from oracle import muon_oracle as O
+    want = O.newton_schulz(G[3].cpu(), O.coefficient_schedule("quintic", 5), 1e-7, storage="fp32")
+    assert _rel(alone, want) <= NS_TOL
