@@ -195,13 +195,16 @@ def require_cuda(t: torch.Tensor, what: str) -> None:
 
 
 # ---------------------------------------------------------------------------
-# workspace: one growing byte buffer per (device, tag); torch owns the memory
+# workspace: one growing byte buffer per (device, stream, tag); torch owns the memory.  The stream is part of the key
+# because torch's allocator orders the reuse of a freed block only against the stream it was allocated on.
 # ---------------------------------------------------------------------------
-_workspaces: Dict[Tuple[int, str], torch.Tensor] = {}
+_workspaces: Dict[Tuple[int, int, str], torch.Tensor] = {}
 
 
 def workspace(device: torch.device, nbytes: int, tag: str = "ns") -> torch.Tensor:
-    key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
+    """Scratch bytes for library calls issued on the current stream of ``device``."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(device).cuda_stream, tag)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
