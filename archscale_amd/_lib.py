@@ -23,6 +23,7 @@ RETRACT_HARD, RETRACT_DYNAMIC = 0, 1
 SN_TRANSPOSED = 1
 NS_CAST_INPUT_FIRST = 1
 NS_NO_NORMALIZE = 2
+NS_NO_DIAG_FOLD = 4
 CHUNK_ELEMS = 8192
 ABI_VERSION = 2
 
@@ -246,7 +247,8 @@ def profile_begin() -> None:
 
 def profile_collect(capacity: int = 4096):
     """Per-launch records of the Newton-Schulz GEMMs since profile_begin():
-    list of dicts {ms, tile, mode, split, final, flops_algorithmic, flops_issued}."""
+    list of dicts {ms, tile, mode, split, final, folded, flops_algorithmic, flops_issued}; ``folded`` marks the
+    X' = (B + aI) X launches that read no addend."""
     ms = (ctypes.c_float * capacity)()
     key = (ctypes.c_int32 * capacity)()
     fa = (ctypes.c_double * capacity)()
@@ -257,6 +259,6 @@ def profile_collect(capacity: int = 4096):
     out = []
     for i in range(min(n, capacity)):
         k = key[i]
-        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool((k % 10) & 2), final=bool((k % 10) & 1),
+        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool((k % 10) & 2), final=bool((k % 10) & 1), folded=bool((k % 10) & 4),
                         flops_algorithmic=fa[i], flops_issued=fi[i]))
     return out

@@ -94,7 +94,7 @@ int compute_units() {
 // one pair of HIP events around every GEMM launch, on the stream the kernel runs on.
 struct ProfRec {
   hipEvent_t start, stop;
-  int key;  // tile*100 + mode*10 + split*2 + final
+  int key;  // tile*100 + mode*10 + 4*(BX without addend) + split*2 + final
   double flops_algorithmic, flops_issued;
 };
 std::mutex g_prof_mutex;
@@ -106,7 +106,7 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
   if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   ProfRec r;
-  r.key = tile * 100 + mode * 10 + (split ? 2 : 0) + (final_ ? 1 : 0);
+  r.key = tile * 100 + mode * 10 + ((mode == MODE_BX && !g.g[0].E) ? 4 : 0) + (split ? 2 : 0) + (final_ ? 1 : 0);
   r.flops_algorithmic = flops_algorithmic;
   r.flops_issued = flops_issued;
   hipError_t e;
@@ -240,7 +240,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   const bool split_any = prec_mode == MUON_PREC_BF16_BSPLIT;
   const int split_tail = (flags >> 8) & 0xff;   // 0: every iteration keeps B as a hi+lo pair; t: only the last t
-  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | MUON_NS_NO_NORMALIZE | 0xff00)) return MUON_E_ARG;
+  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | MUON_NS_NO_NORMALIZE | MUON_NS_NO_DIAG_FOLD | 0xff00)) return MUON_E_ARG;
   const bool normalize = !(flags & MUON_NS_NO_NORMALIZE);
   if (!normalize && fused) return MUON_E_ARG;
   bool split = split_any;
@@ -376,6 +376,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const float a = abc_host[3 * it], b = abc_host[3 * it + 1], c = abc_host[3 * it + 2];
     const bool last = it == iters - 1;
     split = split_any && (split_tail == 0 || it >= iters - split_tail);
+    // a*I folded into B (diagonal entries of B + aI are rounded like any other entry): X' = (B + aI) X needs no addend.
+    // Not for a large `a` (first row of the polar-express table), whose rounding on the diagonal would show.
+    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && fabsf(a) <= 4.2f;
     // A = X X^T, from X^T (K-major operand)
     e = run_mode(MODE_SYRKT, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;
@@ -399,6 +402,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.E = P.A; g.strideE = as; g.lde = pl.Mp;
       g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp; g.alpha = c; g.beta = b;
+      g.diag_add = fold ? a : 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
@@ -412,7 +416,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.P = P.Bh; g.P2 = P.Bl; g.Q = P.Xt[cur]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp;
       g.K = pl.Mp;
       g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
-      g.E = P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
+      g.E = fold ? nullptr : P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
       g.alpha = a; g.beta = 0.f;
       g.scale = (fused && it == 0) ? P.scale : nullptr;
       if (!last) {

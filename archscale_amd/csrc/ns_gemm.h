@@ -18,7 +18,7 @@ struct GemmParams {
   int K;             // reduction length, multiple of 64
   int tilesM, tilesN;
   int batch;
-  const __bf16* E;   // epilogue addend, read as E[col][row..row+3]
+  const __bf16* E;   // epilogue addend, read as E[col][row..row+3]; MODE_BX: may be null (X' = B X, no addend)
   long strideE;
   int lde;
   __bf16* C;         // row-major output [row][col] (may be null in MODE_BX)
@@ -29,6 +29,7 @@ struct GemmParams {
   long strideCt;
   int ldct;
   float alpha, beta;
+  float diag_add;        // MODE_SYRK2: added to the diagonal of the result (B + a I, so that B X needs no addend)
   const float* scale;    // per batch element, or null: SYRK / SYRKT multiply the product by scale^2, BX the result by scale
   int m_valid, n_valid;  // true extents for the bounds-checked final store
   int qt_first;          // quarter mode: first tile of this problem (in its own 2x coarser enumeration) that is covered

@@ -2,8 +2,9 @@
 //
 // The iteration  X <- aX + (bA + cA^2)X,  A = X X^T  keeps ONLY the transposed iterate X^T ([n_long][m]):
 //   SYRKT  A  = X  * X^T         P = Q = X^T, a K-MAJOR operand ([k][m]); fragments by LDS transpose reads
-//   SYRK2  B  = c*A*A + b*A      P = Q = A   (A symmetric, K-contiguous)
-//   BX     X' = a*X + B*X        P = B (symmetric), Q = X^T (K-contiguous); writes X'^T (and X' only for the caller)
+//   SYRK2  B  = c*A*A + b*A      P = Q = A   (A symmetric, K-contiguous); optionally + a*I on the diagonal
+//   BX     X' = a*X + B*X        P = B (symmetric), Q = X^T (K-contiguous); writes X'^T (and X' only for the caller);
+//                                ADDEND = false: X' = B*X for a B that already carries a*I (no X tile in the epilogue)
 // SYRK and SYRK2 compute upper-triangle tiles and mirror them.  SYRK (P = Q = X, K-contiguous) is the stand-alone
 // symmetric rank-k product.  All modes share one main loop (replaces ns_line_1/ns_line_2 and the cuBLAS addmm of
 // lit_gpt/optim/newton_schulz_triton.py:66-139, 181-266, 371-378 and the bf16 SYRK of
@@ -55,7 +56,7 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
 // 16-byte bank groups (rows alternate between the two 128-byte halves of the 64 banks).
 __device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * ROW_BYTES + ((c ^ ((r >> 1) & 7)) << 4); }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL>
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
 ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr int NW = (BM / WM) * (BN / WN);
@@ -404,7 +405,9 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     auto w_off = [&](int c, int r) { return c * WROW + ((((r >> 3) ^ sw(c)) & (RCH - 1)) << 4) + ((r & 7) << 1); };
     const int wrow0 = R0 + wr0, wcol0 = C0 + wc0;  // global origin of this wave's sub-tile
 
-    if (!SYRK_PLAIN) {
+    // MODE_BX without an addend (ADDEND = false): a*I was folded into B's diagonal by the product that made B
+    constexpr bool has_e = !SYRK_PLAIN && (MODE != MODE_BX || ADDEND);
+    if constexpr (has_e) {
       const char* Eb = (const char*)(p.E + (size_t)b * p.strideE + (size_t)wcol0 * p.lde + wrow0);
 #pragma unroll
       for (int t = 0; t < WSLABS; ++t) {
@@ -414,6 +417,16 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    if constexpr (MODE == MODE_BX && !has_e) {
+      if (sc != 1.f) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= sc;
+      }
+    } else
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -576,6 +589,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
             acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
             acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
             acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
+            // diagonal of the matrix (this path runs on diagonal tiles only: R0 == C0)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              if (rl + q == cl) acc[i][j][4 * g + q] += p.diag_add;
           } else {
             acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * sc;
             acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * sc;
@@ -664,11 +681,11 @@ long ns_gemm_tiles(int mode, const GemmParams& p) {
   return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL>
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true>
 static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
-  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL>;
+  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND>;
   // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device
   // (idempotent; a benign race only repeats the call)
   static bool attr_set[64] = {};
@@ -698,11 +715,18 @@ static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGem
       return split ? launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s)
                    : launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false>(p, s);
     case MODE_BX:
+      if (p.g[0].E) {
+        if (split)
+          return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
+                        : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
+        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true>(p, s)
+                      : launch_one<BM, BN, WM, WN, MODE_BX, false, false>(p, s);
+      }
       if (split)
-        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
-                      : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
-      return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true>(p, s)
-                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false>(p, s);
+        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true, false>(p, s)
+                      : launch_one<BM, BN, WM, WN, MODE_BX, true, false, false>(p, s);
+      return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, false>(p, s)
+                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false>(p, s);
   }
   return hipErrorInvalidValue;
 }
@@ -714,6 +738,8 @@ hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, c
   for (int i = 0; i < gp.n_groups; ++i) {
     const GemmParams& g = gp.g[i];
     if (g.K % BK != 0 || g.K <= 0 || gp.tile_start[i + 1] < gp.tile_start[i]) return hipErrorInvalidValue;
+    if (mode == MODE_SYRK2 && !g.E) return hipErrorInvalidValue;
+    if (mode == MODE_BX && (g.E == nullptr) != (gp.g[0].E == nullptr)) return hipErrorInvalidValue;  // one kernel per launch
     // every block must decode to a tile inside the problem
     const long blocks = (long)gp.tile_start[i + 1] - gp.tile_start[i];
     if (!gp.quarter) {

@@ -75,6 +75,7 @@ def newton_schulz(
     out: Optional[Tensor] = None,
     bsplit_tail: int = 0,
     normalize: bool = True,
+    diag_fold: bool = True,
 ) -> Tensor:
     """Orthogonalise every matrix of ``G`` (``[..., rows, cols]``, bf16 or fp32) with the quintic
     Newton-Schulz iteration ``X <- aX + (bA + cA^2)X, A = XX^T``, one ``(a, b, c)`` row per iteration.
@@ -83,7 +84,8 @@ def newton_schulz(
     ``prec="bsplit"`` keeps ``B = bA + cA^2`` as a bf16 hi+lo pair (about +13% work) and is what the
     constant-coefficient table needs to stay within 1e-2 of an fp32 run; ``bsplit_tail=t`` does so only in the
     last ``t`` iterations (0 = all), whose rounding dominates the error of the result.  ``normalize=False`` iterates on
-    the input as it is (``epsilon`` is then unused).
+    the input as it is (``epsilon`` is then unused).  ``diag_fold=False`` keeps ``aX`` as a separate addend in every
+    iteration instead of storing ``B + aI`` where ``|a| <= 4.2``.
     """
     _lib.require_cuda(G, "Newton-Schulz input")
     if G.dtype not in (torch.bfloat16, torch.float32):
@@ -104,6 +106,8 @@ def newton_schulz(
     flags = (_lib.NS_CAST_INPUT_FIRST if cast_input_first else 0) | _lib.ns_bsplit_tail(bsplit_tail)
     if not normalize:
         flags |= _lib.NS_NO_NORMALIZE
+    if not diag_fold:
+        flags |= _lib.NS_NO_DIAG_FOLD
     with torch.cuda.device(G.device):
         st = L.muon_ns_batched(
             Gv.data_ptr(), _lib.dtype_code(Gv.dtype), bstride, ld,

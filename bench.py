@@ -173,14 +173,15 @@ def main():
     # dominant kernel: the X' = aX + BX product in its main (non-final) instantiation
     by_kernel = {}
     for r in recs:
-        k = (r["tile"], r["mode"], r["split"], r["final"])
+        k = (r["tile"], r["mode"], r["split"], r["final"], r["folded"])
         d = by_kernel.setdefault(k, dict(n=0, ms=0.0, fa=0.0, fi=0.0))
         d["n"] += 1; d["ms"] += r["ms"]; d["fa"] += r["flops_algorithmic"]; d["fi"] += r["flops_issued"]
     names = {0: "syrk", 1: "syrk2", 2: "bx", 3: "syrk"}
     kernels = []
-    for (tile, mode, split, final), d in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ms"]):
+    for (tile, mode, split, final, folded), d in sorted(by_kernel.items(), key=lambda kv: -kv[1]["ms"]):
         kernels.append({
             "kernel": f"ns_gemm<{tile},{names[mode]}{',split' if split else ''}{',final' if final else ''}>",
+            "addend": (not folded) if mode == 2 else None,
             "launches_per_step": d["n"], "avg_ms": round(d["ms"] / d["n"], 4),
             "algorithmic_tflops": round(d["fa"] / d["ms"] / 1e9, 1), "issued_tflops": round(d["fi"] / d["ms"] / 1e9, 1),
             "ms_per_step": round(d["ms"], 3)})
@@ -199,8 +200,9 @@ def main():
     }
     if args.layers == N_LAYERS:
         roofline["traffic"] = measured_traffic(roofline["kernel"])
-    if dom_key[1] == 2:  # B (m^2), X^T read twice (operand + addend), X'^T written (X' too by the final launch): bf16
-        per = [(min(s) ** 2 + 3 * min(s) * max(s)) * 2.0 for s in shapes]
+    if dom_key[1] == 2:  # B (m^2), X^T read (once more as the addend unless a*I is folded into B), X'^T written: bf16
+        reads_x = 1 if dom_key[4] else 2
+        per = [(min(s) ** 2 + (reads_x + 1) * min(s) * max(s)) * 2.0 for s in shapes]
         roofline["algorithmic_bytes_per_launch"] = sum(per) * (4 if not dom_key[3] else 1) / dom["n"]
     gemm_ms = sum(d["ms"] for d in by_kernel.values())
     f_issued = sum(d["fi"] for d in by_kernel.values())

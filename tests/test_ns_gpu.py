@@ -229,3 +229,21 @@ def test_quartered_tail_matches_other_grids(ns, gpu_device):
     from oracle import muon_oracle as O
     want = O.newton_schulz(G[3].cpu(), O.coefficient_schedule("quintic", 5), 1e-7, storage="fp32")
     assert _rel(alone, want) <= NS_TOL
+
+
+@pytest.mark.parametrize("table,prec", [("quintic", "bf16"), ("simple", "bsplit"), ("msign", "bsplit")])
+def test_diagonal_fold_and_addend_agree(ns, gpu_device, table, prec):
+    """By default an iteration with |a| <= 4.2 stores B + aI and computes X' = (B + aI) X; diag_fold=False keeps aX as
+    an addend. Both stay within the bar of the fp32 run (their rounding errors are independent of each other)."""
+    G = _randn((2, 512, 1280), 23)
+    coeffs = O.coefficient_schedule(table, 5)
+    kw = dict(prec=prec, bsplit_tail=3 if prec == "bsplit" else 0, eps_mode="clamp" if table == "msign" else "add")
+    folded = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, **kw)
+    addend = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, diag_fold=False, **kw)
+    torch.cuda.synchronize()
+    for b in range(2):
+        want = O.newton_schulz(G[b], coeffs, 1e-7, storage="fp32", eps_mode=kw["eps_mode"])
+        assert _rel(folded[b], want) <= NS_TOL
+        assert _rel(addend[b], want) <= NS_TOL
+        assert _rel(folded[b], addend[b]) <= NS_TOL
+    assert not torch.equal(folded, addend)      # the flag reaches the kernels
