@@ -377,8 +377,10 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const bool last = it == iters - 1;
     split = split_any && (split_tail == 0 || it >= iters - split_tail);
     // a*I folded into B (diagonal entries of B + aI are rounded like any other entry): X' = (B + aI) X needs no addend.
-    // Not for a large `a` (first row of the polar-express table), whose rounding on the diagonal would show.
-    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && fabsf(a) <= 4.2f;
+    // Not for a large `a` (first row of the polar-express table), whose rounding on the diagonal would show, and not in
+    // the first iteration: a matrix with a few dominant singular values has a tiny A after the normalisation, and
+    // B_ii would vanish below half an ulp of `a`.
+    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f;
     // A = X X^T, from X^T (K-major operand)
     e = run_mode(MODE_SYRKT, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;

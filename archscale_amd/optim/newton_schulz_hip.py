@@ -85,7 +85,7 @@ def newton_schulz(
     constant-coefficient table needs to stay within 1e-2 of an fp32 run; ``bsplit_tail=t`` does so only in the
     last ``t`` iterations (0 = all), whose rounding dominates the error of the result.  ``normalize=False`` iterates on
     the input as it is (``epsilon`` is then unused).  ``diag_fold=False`` keeps ``aX`` as a separate addend in every
-    iteration instead of storing ``B + aI`` where ``|a| <= 4.2``.
+    iteration instead of storing ``B + aI`` in the iterations after the first with ``|a| <= 4.2``.
     """
     _lib.require_cuda(G, "Newton-Schulz input")
     if G.dtype not in (torch.bfloat16, torch.float32):

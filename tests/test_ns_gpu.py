@@ -233,7 +233,7 @@ def test_quartered_tail_matches_other_grids(ns, gpu_device):
 
 @pytest.mark.parametrize("table,prec", [("quintic", "bf16"), ("simple", "bsplit"), ("msign", "bsplit")])
 def test_diagonal_fold_and_addend_agree(ns, gpu_device, table, prec):
-    """By default an iteration with |a| <= 4.2 stores B + aI and computes X' = (B + aI) X; diag_fold=False keeps aX as
+    """By default an iteration after the first with |a| <= 4.2 stores B + aI and computes X' = (B + aI) X; diag_fold=False keeps aX as
     an addend. Both stay within the bar of the fp32 run (their rounding errors are independent of each other)."""
     G = _randn((2, 512, 1280), 23)
     coeffs = O.coefficient_schedule(table, 5)
