@@ -380,7 +380,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     // Not for a large `a` (first row of the polar-express table), whose rounding on the diagonal would show, and not in
     // the first iteration: a matrix with a few dominant singular values has a tiny A after the normalisation, and
     // B_ii would vanish below half an ulp of `a`.
-    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f;
+    // With the hi+lo pair the folded diagonal is exact; an iteration of a split call that keeps B in plain bf16 is not
+    // folded (constant coefficients on small matrices: 8.4e-3 -> 1.1e-2 for 64x129 when it is).
+    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f && (!split_any || split);
     // A = X X^T, from X^T (K-major operand)
     e = run_mode(MODE_SYRKT, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;

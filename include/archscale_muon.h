@@ -42,8 +42,9 @@ extern "C" {
                                       (emerging_optimizers/orthogonalized_optimizers/muon_utils.py:262-287) */
 #define MUON_NS_NO_DIAG_FOLD 4     /* always compute X' = aX + BX with the addend; by default an iteration after the first
                                       with |a| <= 4.2 stores B + aI (the diagonal rounded to bf16 like every other entry
-                                      of B, or kept as the hi+lo pair) and computes X' = (B + aI) X, which saves reading
-                                      X a second time */
+                                      of B; with MUON_PREC_BF16_BSPLIT only in the iterations that keep the hi+lo pair,
+                                      where it is exact) and computes X' = (B + aI) X, which saves reading X a second
+                                      time */
 #define MUON_NS_BSPLIT_TAIL(t) (((t) & 0xff) << 8) /* with MUON_PREC_BF16_BSPLIT: only the last t iterations keep B as a
                                                       hi+lo pair (0 = all); the rounding of B in the last iterations
                                                       dominates the error of the result */
