@@ -411,3 +411,41 @@ def test_emerging_fused_momentum_matches_separate_calls(gpu_device, nesterov):
         assert _rel(m1, m2) <= 2e-3       # second step: the buffers see the slightly different weights through l2
         assert _rel(a - w, b - w) <= 1e-2
         assert _rel(a, b) <= 3e-3
+
+
+def test_random_parameter_sets(gpu_device):
+    """Seeded sweep: parameter sets with ragged 2-D and 3-D shapes, both weight dtypes, plain and MuonH updates, with and
+    without Nesterov, weight decay and the fused momentum path; two steps each against the reference-semantics oracle
+    (fp32 Newton-Schulz on the same bf16 inputs)."""
+    import random
+    from archscale_amd.optim.muon import Muon
+    rng = random.Random(77)
+    dims = [64, 96, 100, 129, 200, 256, 320, 513]
+    for case in range(6):
+        shapes = []
+        for _ in range(rng.choice([3, 5])):
+            r, c = rng.choice(dims), rng.choice(dims)
+            shapes.append((rng.choice([2, 3]), r, c) if rng.random() < 0.3 else (r, c))
+        wdtype = rng.choice([torch.float32, torch.bfloat16])
+        use_muonh, nesterov = case % 2 == 0, case % 3 != 0
+        wd, cautious = [(0.1, False), (0.0, False), (0.1, True)][case % 3]
+        fuse = case % 4 != 3
+        adjust = rng.choice(["spectral_norm", "rms_norm", "clip_norm", None])
+        print("case", case, shapes, wdtype, "muonh", use_muonh, "nesterov", nesterov, "wd", wd, cautious, "fuse", fuse, adjust,
+              flush=True)
+        hp = dict(lr=0.02, mu=0.9, wd=wd, eps=1e-8, nesterov=nesterov, adjust=adjust, cautious=cautious)
+        params = _make(shapes, wdtype, 300 + case, gpu_device)
+        w0 = [p.detach().cpu().clone() for p in params]
+        opt = Muon(params, lr=hp["lr"], mu=hp["mu"], weight_decay=wd, cautious_wd=cautious, epsilon=hp["eps"],
+                   nesterov=nesterov, adjust_lr=adjust, use_muonh=use_muonh, fuse_momentum=fuse)
+        steps = [_grads(shapes, wdtype, 400 + 10 * case + k) for k in range(2)]
+        for grads in steps:
+            for p, g in zip(params, grads):
+                p.grad = g.to(gpu_device)
+            opt.step()
+        torch.cuda.synchronize()
+        Xf, Mf = _oracle_run(shapes, w0, steps, wdtype=wdtype, hp=hp, use_muonh=use_muonh, ns_storage="fp32")
+        for p, xf, mf in zip(params, Xf, Mf):
+            assert torch.isfinite(p.detach().float()).all()
+            assert _rel(p.detach(), xf) <= W_TOL, (case, tuple(p.shape))
+            assert _rel(opt.state[p]["momentum"], mf) <= (1e-6 if wdtype == torch.float32 else 1e-2)
