@@ -112,7 +112,8 @@ void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
  * bracketed by a pair of HIP events on its stream.  muon_profile_collect waits for them, writes up to `capacity`
  * records to the HOST arrays (any may be NULL) and returns the number of launches recorded (< 0 on error):
  *   ms                elapsed milliseconds of the launch
- *   key               tile*100 + mode*10 + split*2 + final  (mode 0 = X X^T, 1 = cAA+bA, 2 = aX + BX)
+ *   key               tile*100 + mode*10 + 4*noaddend + split*2 + final  (mode 0 = X X^T, 1 = cAA+bA, 2 = aX + BX,
+ *                     3 = X X^T from the transposed iterate; noaddend: an X' = (B + aI) X launch)
  *   flops_algorithmic minimum FLOPs of the product (symmetric products counted once)
  *   flops_issued      FLOPs of the tiles actually launched
  */
