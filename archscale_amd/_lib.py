@@ -17,7 +17,7 @@ from .build import LIB_PATH
 # enums of include/archscale_muon.h
 DTYPE_BF16, DTYPE_F32 = 0, 1
 EPS_ADD, EPS_CLAMP = 0, 1
-PREC_BF16, PREC_BF16_BSPLIT = 0, 1
+PREC_BF16, PREC_BF16_BSPLIT, PREC_F16 = 0, 1, 2
 ALGO_ADAMW, ALGO_LION = 0, 1
 RETRACT_HARD, RETRACT_DYNAMIC = 0, 1
 SN_TRANSPOSED = 1

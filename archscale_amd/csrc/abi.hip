@@ -102,8 +102,8 @@ std::vector<ProfRec> g_prof;
 std::atomic<bool> g_prof_on{false};
 
 hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GroupedGemmParams& g, hipStream_t stream,
-                      double flops_algorithmic, double flops_issued) {
-  if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
+                      double flops_algorithmic, double flops_issued, bool f16 = false) {
+  if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16);
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   ProfRec r;
   r.key = tile * 100 + mode * 10 + ((mode == MODE_BX && !g.g[0].E) ? 4 : 0) + (split ? 2 : 0) + (final_ ? 1 : 0);
@@ -116,7 +116,7 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
     (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop);
     return e;
   }
-  e = launch_ns_gemm_grouped(tile, mode, split, final_, g, stream);
+  e = launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16);
   hipError_t e2 = hipEventRecord(r.stop, stream);
   g_prof.push_back(r);
   return e != hipSuccess ? e : e2;
@@ -131,18 +131,18 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
 // is quartered as a whole up to QUARTER_MAX_ALONE tiles.  ARCHSCALE_MUON_QUARTER=0 switches it off.
 constexpr int QUARTER_MAX_TAIL = 128, QUARTER_MAX_ALONE = 176;
 hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp, hipStream_t stream,
-                         double fa, double fi) {
+                         double fa, double fi, bool f16) {
   static const bool enabled = !(getenv("ARCHSCALE_MUON_QUARTER") && atoi(getenv("ARCHSCALE_MUON_QUARTER")) == 0);
   const int total = gp.tile_start[gp.n_groups];
   const int round = 256;
   const int full = total / round * round, tail = total - full;
   if (!enabled || tile != 256 || tail == 0 || tail > (full > 0 ? QUARTER_MAX_TAIL : QUARTER_MAX_ALONE))
-    return timed_gemm(tile, mode, split, final_, gp, stream, fa, fi);
+    return timed_gemm(tile, mode, split, final_, gp, stream, fa, fi, f16);
   const double share = (double)full / total;
   if (full > 0) {
     GroupedGemmParams m = gp;
     for (int i = 0; i <= gp.n_groups; ++i) m.tile_start[i] = std::min(gp.tile_start[i], full);
-    hipError_t e = timed_gemm(tile, mode, split, final_, m, stream, fa * share, fi * share);
+    hipError_t e = timed_gemm(tile, mode, split, final_, m, stream, fa * share, fi * share, f16);
     if (e != hipSuccess) return e;
   }
   GroupedGemmParams q = {};
@@ -159,7 +159,7 @@ hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const Grou
     q.tile_start[q.n_groups + 1] = q.tile_start[q.n_groups] + 4 * (e - f);
     ++q.n_groups;
   }
-  return timed_gemm(128, mode, split, final_, q, stream, fa * (1.0 - share), fi * (1.0 - share));
+  return timed_gemm(128, mode, split, final_, q, stream, fa * (1.0 - share), fi * (1.0 - share), f16);
 }
 
 }  // namespace
@@ -204,6 +204,7 @@ struct NsProblem {
   __bf16 *Xt[2], *A, *Bh, *Bl;   // Xt: the iterate as X^T, [b][Np][Mp] (long side first), ping-pong
   float *partial, *scale;
   bool tall;
+  int sx;   // half-precision mode: the iterate is kept times 2^sx (its rms entry starts at about 2^-3)
 };
 
 int check_problem(const muon_ns_problem& q, bool no_input = false) {
@@ -236,7 +237,10 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   hipStream_t stream = (hipStream_t)stream_;
   if (!problems_host || n_problems <= 0 || !abc_host || !ws_dev || iters <= 0) return MUON_E_ARG;
   if (eps_mode != MUON_EPS_ADD && eps_mode != MUON_EPS_CLAMP) return MUON_E_ARG;
-  if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT) return MUON_E_ARG;
+  if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT && prec_mode != MUON_PREC_F16) return MUON_E_ARG;
+  const bool f16 = prec_mode == MUON_PREC_F16;
+  // power-of-two factors of the half-precision workspace: A is kept times 2^SA, B times 2^SB, X times 2^sx (per problem)
+  const int SA = f16 ? 8 : 0, SB = f16 ? 6 : 0;
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   const bool split_any = prec_mode == MUON_PREC_BF16_BSPLIT;
   const int split_tail = (flags >> 8) & 0xff;   // 0: every iteration keeps B as a hi+lo pair; t: only the last t
@@ -276,6 +280,11 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     P.partial = (float*)(ws + P.pl.off_partial);
     P.scale = (float*)(ws + P.pl.off_scale);
     P.tall = P.q.rows > P.q.cols;
+    P.sx = 0;
+    if (f16) {
+      const int l2 = (int)floor(0.5 * log2((double)P.pl.m * (double)P.pl.n)) - 3;
+      P.sx = l2 > 0 ? l2 : 0;
+    }
   }
   // launch order inside a grouped kernel: problems with the longest tiles first, so the tail of the
   // grid is made of short tiles
@@ -299,10 +308,10 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     }
     if (!P.tall)
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, sc, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream);
+                        P.q.cols, sc, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream, f16, P.sx);
     else
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream);
+                        P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream, f16, P.sx);
     if (e != hipSuccess) return (int)e;
   }
   // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials
@@ -332,6 +341,13 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     }
     e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);
     if (e != hipSuccess) return (int)e;
+    if (f16) {
+      // the unnormalised bfloat16 update cannot go into half as it is (its magnitude is the gradient's): one pass in
+      // place turns it into half(2^sx * X / |X|); the deferred scale of the bfloat16 path is then not used
+      e = launch_layout(P.Xt[0], MUON_DTYPE_BF16, 0, xs, pl.Mp, P.q.batch, pl.Np, pl.Mp, P.scale, P.Xt[0], xs, pl.Mp,
+                        pl.Np, pl.Mp, nullptr, 0, 0, stream, 1, P.sx);
+      if (e != hipSuccess) return (int)e;
+    }
   }
 
   // one product of the iteration for every problem: problems that share a tile configuration go into one
@@ -342,7 +358,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       double fa = 0.0, fi = 0.0;
       auto flush = [&]() -> hipError_t {
         if (gp.n_groups == 0) return hipSuccess;
-        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi);
+        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi, f16);
         gp = GroupedGemmParams{};
         fa = fi = 0.0;
         return err;
@@ -390,8 +406,8 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.batch = P.q.batch;
       g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
-      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
-      g.scale = (fused && it == 0) ? P.scale : nullptr;
+      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, SA - 2 * P.sx); g.beta = 0.f;
+      g.scale = (fused && it == 0 && !f16) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
@@ -405,8 +421,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.P = P.A; g.Q = P.A; g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.E = P.A; g.strideE = as; g.lde = pl.Mp;
-      g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp; g.alpha = c; g.beta = b;
-      g.diag_add = fold ? a : 0.f;
+      g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp;
+      g.alpha = ldexpf(c, SB - 2 * SA); g.beta = ldexpf(b, SB - SA);
+      g.diag_add = fold ? ldexpf(a, SB) : 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
@@ -421,8 +438,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.K = pl.Mp;
       g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
       g.E = fold ? nullptr : P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
-      g.alpha = a; g.beta = 0.f;
-      g.scale = (fused && it == 0) ? P.scale : nullptr;
+      g.alpha = ldexpf(a, SB); g.beta = 0.f;
+      g.out_shift = -SB - (last ? P.sx : 0);   // the caller's result is the iterate itself, without its factor
+      g.scale = (fused && it == 0 && !f16) ? P.scale : nullptr;
       if (!last) {
         g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {

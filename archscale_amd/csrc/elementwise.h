@@ -40,7 +40,7 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
 // d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).
 hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
-                         void* T, long t_bstride, int ldt, hipStream_t stream);
+                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16 = 0, int out_shift = 0);
 
 // momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
 constexpr int MOMLAY_MAX = 32;

@@ -228,7 +228,7 @@ norm_scale_kernel(const float* __restrict__ partial, int chunks_per_mat, float e
 }
 
 // ---------------------------------------------------------------------------
-// 3. normalise + lay out:  D[b][r][c] = bf16(s_b * in[b][r][c]),  T[b][c][r] = same value,
+// 3. normalise + lay out:  D[b][r][c] = bf16(s_b * in[b][r][c]) (or half(2^shift * s_b * in)),  T[b][c][r] = same value,
 //    both zero-padded to the tile multiples the GEMMs assume (replaces the
 //    X/(norm+eps), .mT and .contiguous() of newton_schulz_triton.py:358-366).
 // ---------------------------------------------------------------------------
@@ -237,13 +237,14 @@ __global__ void __launch_bounds__(256)
 normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, int cols, int ld,
                         const float* __restrict__ scale,
                         uint16_t* __restrict__ D, long d_bstride, int ldd, int d_rows, int d_cols,
-                        uint16_t* __restrict__ T, long t_bstride, int ldt) {
+                        uint16_t* __restrict__ T, long t_bstride, int ldt, int out_f16, int out_shift) {
   // 64x64 tile; d_rows/d_cols are the padded extents (multiples of 64)
   __shared__ uint16_t tile[64][66];
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const char* base = (const char*)in + (size_t)b * in_bstride * sizeof(typename Elem<DT>::T);
   const float s = scale ? scale[b] : 1.f;
+  const float fs = __builtin_ldexpf(1.f, out_shift);
   const int tr = threadIdx.x >> 3;        // 0..31
   const int tc = (threadIdx.x & 7) * 8;   // 0..56
   const bool vec = aligned16(base) && (ld % 8 == 0) && (in_bstride % 8 == 0);
@@ -261,7 +262,8 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const float x = CAST_FIRST ? bf2f(f2bf(v[k])) : v[k];
-      o[k] = f2bf(x * s);
+      // half output: times 2^out_shift, which keeps the normalised entries in the normal range of the format
+      o[k] = out_f16 ? __builtin_bit_cast(uint16_t, (_Float16)(x * s * fs)) : f2bf(x * s);
       tile[tr + h * 32][tc + k] = o[k];
     }
     if (D && r < d_rows && c < d_cols) {
@@ -310,12 +312,13 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
 
 hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
-                         void* T, long t_bstride, int ldt, hipStream_t stream) {
+                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16, int out_shift) {
   if (batch > 65535 || d_rows / 64 > 65535 || d_rows % 64 || d_cols % 64) return hipErrorInvalidValue;
   dim3 g3(d_cols / 64, d_rows / 64, batch);
 #define ARCHSCALE_NL(DT, CF)                                                                                   \
   hipLaunchKernelGGL((normalize_layout_kernel<DT, CF>), g3, dim3(256), 0, stream, in, in_bstride, rows, cols,  \
-                     ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride, ldt)
+                     ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride, ldt,    \
+                     out_f16, out_shift)
   if (in_dtype == DT_BF16) ARCHSCALE_NL(DT_BF16, false);
   else if (cast_first) ARCHSCALE_NL(DT_F32, true);
   else ARCHSCALE_NL(DT_F32, false);

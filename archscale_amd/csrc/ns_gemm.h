@@ -29,6 +29,7 @@ struct GemmParams {
   long strideCt;
   int ldct;
   float alpha, beta;
+  int out_shift;         // MODE_BX: the result is multiplied by 2^out_shift (0: as it is)
   float diag_add;        // MODE_SYRK2: added to the diagonal of the result (B + a I, so that B X needs no addend)
   const float* scale;    // per batch element, or null: SYRK / SYRKT multiply the product by scale^2, BX the result by scale
   int m_valid, n_valid;  // true extents for the bounds-checked final store
@@ -53,8 +54,9 @@ struct GroupedGemmParams {
 long ns_gemm_tiles(int mode, const GemmParams& p);
 
 // tile: 256 (256x256 block tile, 8 waves) or 128 (128x128, 4 waves)
+// f16: the workspace matrices of the launch are IEEE half (see GemmParams::out_shift); not with split
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
-                                  hipStream_t stream);
+                                  hipStream_t stream, bool f16 = false);
 hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream);
 
 }  // namespace archscale

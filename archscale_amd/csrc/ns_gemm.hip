@@ -44,6 +44,10 @@ __device__ __forceinline__ uint16_t bf16_bits(float f) {
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
+__device__ __forceinline__ uint16_t f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+__device__ __forceinline__ float f16_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
 __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
   uint2 r;
   r.x = (uint32_t)bf16_bits(a) | ((uint32_t)bf16_bits(b) << 16);
@@ -56,9 +60,12 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
 // 16-byte bank groups (rows alternate between the two 128-byte halves of the 64 banks).
 __device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * ROW_BYTES + ((c ^ ((r >> 1) & 7)) << 4); }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND>
+// F16: the workspace matrices (operands, addend, non-final outputs) are IEEE half instead of bfloat16 (the caller's
+// tensors stay bfloat16); the host keeps them in range with power-of-two factors folded into alpha / beta / out_shift.
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND, bool F16>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
 ns_gemm_kernel(const GroupedGemmParams gp) {
+  static_assert(!(F16 && SPLIT), "the hi+lo pair is a bfloat16 device");
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int WAVES_N = BN / WN;
   constexpr int FM = WM / 32, FN = WN / 32;
@@ -72,6 +79,15 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   constexpr bool SYM = (SYRK_PLAIN || MODE == MODE_SYRK2);
   // SPLIT means "B is a hi+lo pair": SYRK2 WRITES the pair, BX READS it as a second pass over K
   constexpr bool KSPLIT = SPLIT && MODE == MODE_BX;
+  // element codecs: workspace data is half or bfloat16; the final launch writes the caller's bfloat16
+  auto dec = [](uint32_t bits) { return F16 ? f16_to_f32((uint16_t)bits) : bf16_to_f32((uint16_t)bits); };
+  auto enc = [](float f) { return (F16 && !FINAL) ? f16_bits(f) : bf16_bits(f); };
+  auto pk4 = [&](float a, float b, float c, float d) {
+    uint2 r;
+    r.x = (uint32_t)enc(a) | ((uint32_t)enc(b) << 16);
+    r.y = (uint32_t)enc(c) | ((uint32_t)enc(d) << 16);
+    return r;
+  };
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -260,7 +276,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
     for (int q = 0; q < NMF; ++q) {
       if (COMPUTE)
-        acc[q / FN][q % FN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cbuf][q / FN], bq[cbuf][q % FN], acc[q / FN][q % FN], 0, 0, 0);
+        acc[q / FN][q % FN] = F16 ? __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[cbuf][q / FN]), __builtin_bit_cast(f16x8, bq[cbuf][q % FN]), acc[q / FN][q % FN], 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cbuf][q / FN], bq[cbuf][q % FN], acc[q / FN][q % FN], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
       const int g_lo = g0 + (q * (g1 - g0) + NMF - 1) / NMF, g_hi = g0 + ((q + 1) * (g1 - g0) + NMF - 1) / NMF;
       if (READ && q < NRD) fread(rbuf, rP, rQ, rkk, q);
@@ -347,6 +364,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   // optional per-matrix scale of the operand that was left out of it (deferred normalisation): the product of two
   // such operands carries sc^2, a product with one of them (and its addend) carries sc
   const float sc = p.scale ? p.scale[b] : 1.f;
+  const float bx_sc = sc * __builtin_ldexpf(1.f, p.out_shift);   // MODE_BX: scale of the result (a power of two from the host)
   const float alpha = SYRK_PLAIN ? p.alpha * sc * sc : p.alpha, beta = p.beta;
   const bool diag = SYM && (ti == tj);
   // S[cl][rl]: chunk index XOR cl, so the 32 lanes of an 8-byte access (32 different cl) spread over all banks
@@ -418,13 +436,13 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     if constexpr (MODE == MODE_BX && !has_e) {
-      if (sc != 1.f) {
+      if (bx_sc != 1.f) {
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
           for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] *= sc;
+            for (int e = 0; e < 16; ++e) acc[i][j][e] *= bx_sc;
       }
     } else
 #pragma unroll
@@ -440,18 +458,18 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
             for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
           } else {
             const uint2 e = *(const uint2*)(W + w_off(c, r));
-            const float e0 = bf16_to_f32(e.x & 0xffff), e1 = bf16_to_f32(e.x >> 16);
-            const float e2 = bf16_to_f32(e.y & 0xffff), e3 = bf16_to_f32(e.y >> 16);
+            const float e0 = dec(e.x & 0xffff), e1 = dec(e.x >> 16);
+            const float e2 = dec(e.y & 0xffff), e3 = dec(e.y >> 16);
             if (MODE == MODE_SYRK2) {
               acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
               acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
               acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
               acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
             } else {
-              acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * sc;
-              acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * sc;
-              acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * sc;
-              acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * sc;
+              acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * bx_sc;
+              acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * bx_sc;
+              acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * bx_sc;
+              acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * bx_sc;
             }
           }
         }
@@ -467,7 +485,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
           for (int g = 0; g < 4; ++g)
             *(uint2*)(W + w_off(j * 32 + l32, i * 32 + 8 * g + 4 * hi)) =
-                pack4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                pk4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
       // transposed / mirrored image: rows of W
       __bf16* Tdst = SYM ? Cdst : p.Ct;
       if (Tdst) {
@@ -582,8 +600,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
           for (int q = 0; q < 4; ++q) acc[i][j][4 * g + q] *= alpha;
         } else {
           const uint2 e = *(const uint2*)(smem + s_off(cl, rl));
-          const float e0 = bf16_to_f32(e.x & 0xffff), e1 = bf16_to_f32(e.x >> 16);
-          const float e2 = bf16_to_f32(e.y & 0xffff), e3 = bf16_to_f32(e.y >> 16);
+          const float e0 = dec(e.x & 0xffff), e1 = dec(e.x >> 16);
+          const float e2 = dec(e.y & 0xffff), e3 = dec(e.y >> 16);
           if (MODE == MODE_SYRK2) {
             acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
             acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
@@ -594,10 +612,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
             for (int q = 0; q < 4; ++q)
               if (rl + q == cl) acc[i][j][4 * g + q] += p.diag_add;
           } else {
-            acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * sc;
-            acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * sc;
-            acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * sc;
-            acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * sc;
+            acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * bx_sc;
+            acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * bx_sc;
+            acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * bx_sc;
+            acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * bx_sc;
           }
         }
       }
@@ -619,7 +637,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
           for (int g = 0; g < 4; ++g) {
             const int rl = wr0 + i * 32 + 8 * g + 4 * hi;
             *(uint2*)(smem + s_off(cl, rl)) =
-                pack4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                pk4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
           }
         }
       __syncthreads();
@@ -639,7 +657,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int rl = wr0 + i * 32 + 8 * g + 4 * hi + q;
-              const uint16_t bits = bf16_bits(acc[i][j][4 * g + q]);
+              const uint16_t bits = enc(acc[i][j][4 * g + q]);
               if (!diag) {
                 *(uint16_t*)(smem + d_off(rl, cl * 2)) = bits;
               } else if (cl >= rl) {
@@ -681,11 +699,11 @@ long ns_gemm_tiles(int mode, const GemmParams& p) {
   return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true>
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true, bool F16 = false>
 static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
-  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND>;
+  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>;
   // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device
   // (idempotent; a benign race only repeats the call)
   static bool attr_set[64] = {};
@@ -704,35 +722,40 @@ static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool F16>
 static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGemmParams& p, hipStream_t s) {
+  if (F16 && split) return hipErrorInvalidValue;
   switch (mode) {
     case MODE_SYRK:
-      return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false>(p, s);
+      return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false, true, F16>(p, s);
     case MODE_SYRKT:
-      return launch_one<BM, BN, WM, WN, MODE_SYRKT, false, false>(p, s);
+      return launch_one<BM, BN, WM, WN, MODE_SYRKT, false, false, true, F16>(p, s);
     case MODE_SYRK2:
-      return split ? launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s)
-                   : launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false>(p, s);
-    case MODE_BX:
-      if (p.g[0].E) {
-        if (split)
-          return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
-                        : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
-        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true>(p, s)
-                      : launch_one<BM, BN, WM, WN, MODE_BX, false, false>(p, s);
+      if constexpr (!F16) {
+        if (split) return launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s);
       }
-      if (split)
-        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true, false>(p, s)
-                      : launch_one<BM, BN, WM, WN, MODE_BX, true, false, false>(p, s);
-      return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, false>(p, s)
-                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false>(p, s);
+      return launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false, true, F16>(p, s);
+    case MODE_BX:
+      if constexpr (!F16) {
+        if (split) {
+          if (p.g[0].E)
+            return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
+                          : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
+          return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true, false>(p, s)
+                        : launch_one<BM, BN, WM, WN, MODE_BX, true, false, false>(p, s);
+        }
+      }
+      if (p.g[0].E)
+        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, true, F16>(p, s)
+                      : launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, F16>(p, s);
+      return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, false, F16>(p, s)
+                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false, F16>(p, s);
   }
   return hipErrorInvalidValue;
 }
 
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, bool f16) {
   if (gp.n_groups < 1 || gp.n_groups > MAX_GROUPS) return hipErrorInvalidValue;
   const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2 || mode == MODE_SYRKT);
   for (int i = 0; i < gp.n_groups; ++i) {
@@ -751,8 +774,13 @@ hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, c
       if (g.qt_first + blocks / 4 > coarse) return hipErrorInvalidValue;
     }
   }
-  if (tile == 256) return launch_cfg<256, 256, 128, 64>(mode, split, final_, gp, stream);
-  if (tile == 128) return launch_cfg<128, 128, 64, 64>(mode, split, final_, gp, stream);
+  if (f16) {
+    if (tile == 256) return launch_cfg<256, 256, 128, 64, true>(mode, split, final_, gp, stream);
+    if (tile == 128) return launch_cfg<128, 128, 64, 64, true>(mode, split, final_, gp, stream);
+    return hipErrorInvalidValue;
+  }
+  if (tile == 256) return launch_cfg<256, 256, 128, 64, false>(mode, split, final_, gp, stream);
+  if (tile == 128) return launch_cfg<128, 128, 64, 64, false>(mode, split, final_, gp, stream);
   return hipErrorInvalidValue;
 }
 

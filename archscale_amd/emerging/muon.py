@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 from torch.optim.optimizer import ParamsT
 
+from ..optim import newton_schulz_hip as ns
 from .mixin import WeightDecayT
 from .orthogonalized_optimizer import OrthogonalizedOptimizer
 from .spectral_ball_utils import msign, msign_schedule
@@ -70,5 +71,5 @@ class Muon(OrthogonalizedOptimizer):
         if self.scaled_orthogonalize_fn is not self._builtin_fn:
             return None  # someone replaced the hook: honour it per parameter
         mode, extra = self._scale_mode, self._extra_scale_factor
-        return (msign_schedule(self._num_ns_steps), 1e-7, "clamp", "bsplit",
+        return (msign_schedule(self._num_ns_steps), 1e-7, "clamp", ns.ACCURATE_PREC,
                 lambda rows, cols: get_muon_scale_factor(rows, cols, mode=mode) * extra)

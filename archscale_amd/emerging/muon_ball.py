@@ -392,7 +392,7 @@ class MuonBall(OrthogonalizedOptimizer):
                                                 ws.numel(), stream), "muon_spectral_norm")
             # Phi = msign(U) for every piece, written into the bf16 update buffers
             n_ns = len(plan.ns_groups)
-            pm = _lib.PREC_BF16_BSPLIT
+            pm = ns._PREC[ns.ACCURATE_PREC]
             coeffs = msign_schedule(self.msign_steps)
             if base.fused:
                 need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in base.fused_probs)

@@ -60,8 +60,7 @@ def newton_schulz(x: torch.Tensor, steps: int, coefficient_type: str = "polar_ex
     if steps % len(sets) != 0:
         raise ValueError(f"steps ({steps}) must be multiple of len(coefficient_sets) ({len(sets)}).")
     rows = [tuple(sets[i % len(sets)]) for i in range(steps)]
-    out = ns.newton_schulz(x, rows, eps, eps_mode="clamp", prec="bsplit", cast_input_first=False,
-                           bsplit_tail=ns.BSPLIT_TAIL)
+    out = ns.newton_schulz(x, rows, eps, eps_mode="clamp", prec=ns.ACCURATE_PREC, cast_input_first=False)
     return out.to(torch.float32)
 
 

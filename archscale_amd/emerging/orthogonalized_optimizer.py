@@ -223,7 +223,7 @@ class OrthogonalizedOptimizer(WeightDecayMixin, optim.Optimizer):
             um, ug = (beta, 1.0 - beta) if self.use_nesterov else (1.0, 0.0)
             if fused:
                 coeffs, eps, eps_mode, prec, _ = recipe
-                pm = _lib.PREC_BF16_BSPLIT if prec == "bsplit" else _lib.PREC_BF16
+                pm = ns._PREC[prec]
                 em = _lib.EPS_CLAMP if eps_mode == "clamp" else _lib.EPS_ADD
                 need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in plan.fused_probs)
                 ws = _lib.workspace(device, need)

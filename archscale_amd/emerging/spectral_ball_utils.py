@@ -35,8 +35,7 @@ def msign(G: torch.Tensor, steps: int) -> torch.Tensor:
         raise ValueError("Input tensor must have at least 2 dimensions.")
     if G.dtype != torch.float32:
         raise ValueError("Input tensor G must be in float32")
-    return ns.newton_schulz(G, msign_schedule(steps), 1e-7, eps_mode="clamp", prec="bsplit", cast_input_first=False,
-                            bsplit_tail=ns.BSPLIT_TAIL)
+    return ns.newton_schulz(G, msign_schedule(steps), 1e-7, eps_mode="clamp", prec=ns.ACCURATE_PREC, cast_input_first=False)
 
 
 # ---------------------------------------------------------------------------

@@ -236,7 +236,8 @@ class Muon(Optimizer):
 
     Extra keyword-only knobs of this implementation:
       ns_coefficients   (a, b, c) rows, one per iteration (default: the reference's 5-row schedule)
-      ns_precision      "bf16" or "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair)
+      ns_precision      "bf16", "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair) or "f16" (the iteration's matrices
+                        in IEEE half inside the workspace, scaled by powers of two: 8x the mantissa at the same rate)
       muonh_per_matrix  renormalise each matrix of a 3-D parameter on its own instead of the whole tensor
       fuse_momentum     momentum and Newton-Schulz in one library call that never stores the bf16 update in the
                         parameter's orientation (default; falls back to separate calls with a hook or a tight limit)
@@ -277,7 +278,7 @@ class Muon(Optimizer):
             raise ValueError(
                 f"Invalid adjust_lr value: {adjust_lr}. Must be 'spectral_norm', 'rms_norm', 'clip_norm', or None."
             )
-        if ns_precision not in ("bf16", "bsplit"):
+        if ns_precision not in ("bf16", "bsplit", "f16"):
             raise ValueError(f"Invalid ns_precision: {ns_precision}")
 
         defaults = dict(
@@ -438,7 +439,7 @@ class Muon(Optimizer):
         if self._newton_schulz_func is not None or not self._fuse_momentum or plan.fused_probs is None:
             return False
         L = _lib.lib()
-        pm = _lib.PREC_BF16_BSPLIT if self._ns_precision == "bsplit" else _lib.PREC_BF16
+        pm = ns._PREC[self._ns_precision]
         n = len(plan.fused_probs)
         need = sum(L.muon_ns_workspace_bytes(q.batch, q.rows, q.cols, pm) for q in plan.fused_probs)
         if need > self._ns_workspace_limit:
@@ -455,7 +456,7 @@ class Muon(Optimizer):
         """U <- NS(U) for every shape class in ONE grouped call (each product of the iteration is one launch over
         all classes); classes are sliced / the call is split only when the workspace would exceed the limit."""
         L = _lib.lib()
-        pm = _lib.PREC_BF16_BSPLIT if self._ns_precision == "bsplit" else _lib.PREC_BF16
+        pm = ns._PREC[self._ns_precision]
         parts: List[Tensor] = []
         used = 0
 

@@ -33,12 +33,16 @@ QUINTIC_SCHEDULE: Coeffs = (
 #: lit_gpt/legacy_optim.py:198
 SIMPLE_ROW = (3.4445, -4.7750, 2.0315)
 
-_PREC = {"bf16": _lib.PREC_BF16, "bsplit": _lib.PREC_BF16_BSPLIT}
+_PREC = {"bf16": _lib.PREC_BF16, "bsplit": _lib.PREC_BF16_BSPLIT, "f16": _lib.PREC_F16}
 #: iterations (counted from the end) that keep B as a hi+lo pair wherever this package asks for the split itself.
 #: Measured against fp32 runs on the same bf16 input (N(0,1), 256x2048 .. 2048x5632): constant-row table x5
 #: 1.1-1.3e-2 without the split, 7.7-8.3e-3 with the last 2, 6.0-6.8e-3 with the last 3 and with all 5; the
 #: polar-express table x5 8.1-9.2e-3 / 6.9-8.5e-3 / 5.7-7.4e-3 / 5.7-7.3e-3.
 BSPLIT_TAIL = 3
+#: precision mode for the coefficient tables that plain bf16 storage cannot keep within 1e-2 of an fp32 run (constant
+#: coefficients, polar express): the half-precision workspace - one walk per product, a third of the error of the
+#: hi+lo pair
+ACCURATE_PREC = "f16"
 _EPS = {"add": _lib.EPS_ADD, "clamp": _lib.EPS_CLAMP}
 
 
@@ -81,8 +85,10 @@ def newton_schulz(
     Newton-Schulz iteration ``X <- aX + (bA + cA^2)X, A = XX^T``, one ``(a, b, c)`` row per iteration.
 
     Returns a new bf16 tensor shaped like ``G`` (``G`` itself is not modified unless ``out is G``).
-    ``prec="bsplit"`` keeps ``B = bA + cA^2`` as a bf16 hi+lo pair (about +13% work) and is what the
-    constant-coefficient table needs to stay within 1e-2 of an fp32 run; ``bsplit_tail=t`` does so only in the
+    ``prec="f16"`` keeps the iterate and both Gram-side matrices in IEEE half inside the workspace (scaled by powers of
+    two; 8x the mantissa of bf16 at the same matrix-core rate): what the constant-coefficient and polar-express tables
+    need to stay within 1e-2 of an fp32 run.  ``prec="bsplit"`` stays in bf16 and keeps ``B = bA + cA^2`` as a hi+lo
+    pair (a second walk over K in ``BX``); ``bsplit_tail=t`` does so only in the
     last ``t`` iterations (0 = all), whose rounding dominates the error of the result.  ``normalize=False`` iterates on
     the input as it is (``epsilon`` is then unused).  ``diag_fold=False`` keeps ``aX`` as a separate addend in every
     iteration instead of storing ``B + aI`` in the iterations after the first with ``|a| <= 4.2``.
@@ -183,7 +189,7 @@ newton_schulz_triton = newton_schulz_hip
 def zeropower_via_newtonschulz5_legacy(G: Tensor, steps: int = 5) -> Tensor:
     """Drop-in for lit_gpt/legacy_optim.py:187-213: constant (3.4445, -4.7750, 2.0315) row, eps 1e-7."""
     assert G.ndim >= 2
-    return newton_schulz(G, [SIMPLE_ROW] * steps, 1e-7, prec="bsplit", bsplit_tail=BSPLIT_TAIL)
+    return newton_schulz(G, [SIMPLE_ROW] * steps, 1e-7, prec=ACCURATE_PREC)
 
 
 # ---------------------------------------------------------------------------

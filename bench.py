@@ -107,6 +107,8 @@ def main():
     ap.add_argument("--coeffs", choices=["quintic", "simple"], default="quintic",
                     help="quintic = the reference's production 5-row schedule; simple = constant row with the B split")
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="(debug) fewer layers; the result is then not the metric")
+    ap.add_argument("--precision", choices=["bf16", "f16"], default="bf16",
+                    help="storage of the iteration's matrices inside the Newton-Schulz workspace (inputs and outputs stay bf16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--separate-momentum", action="store_true",
                     help="(comparison) momentum kernel and Newton-Schulz as separate library calls instead of the fused one")
@@ -131,7 +133,8 @@ def main():
     simple = args.coeffs == "simple"
     opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, adjust_lr="spectral_norm",
                use_muonh=True, ns_coefficients=[H.SIMPLE_ROW] * 5 if simple else None,
-               ns_precision="bsplit" if simple else "bf16", fuse_momentum=not args.separate_momentum)
+               ns_precision=("f16" if args.precision == "f16" else "bsplit" if simple else "bf16"),
+               fuse_momentum=not args.separate_momentum)
 
     for _ in range(args.warmup):  # also warms the momentum so that M != G
         opt.step()
@@ -222,11 +225,12 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "f16" if args.precision == "f16" else "bf16", "data": "synthetic",
         "config": {"workload": f"config 2: full MuonH step, depth-{args.layers} GQA transformer, "
                                f"{len(params)} bf16 matrices, {n_elem / 1e6:.1f} M elements, "
                                f"mu 0.95 nesterov, NS5 {args.coeffs} coefficients, lr 0.02, seed {args.seed}",
-                   "coefficients": args.coeffs, "ns_precision": "bsplit" if simple else "bf16"},
+                   "coefficients": args.coeffs,
+                   "ns_precision": "f16" if args.precision == "f16" else "bsplit" if simple else "bf16"},
         "value_definition": "dense-count NS FLOPs (5*(4m^2n+2m^3) per matrix) / wall time of the WHOLE step",
         "ns_gemm_pct_mfma_peak_issued": round(f_issued / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
         "ns_gemm_pct_mfma_peak_symmetric": round(f_sym / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),

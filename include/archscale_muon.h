@@ -33,6 +33,10 @@ extern "C" {
 /* precision of B = bA + cA^2 as an operand of B*X */
 #define MUON_PREC_BF16 0       /* one bf16 rounding per GEMM epilogue (rounding points of newton_schulz_triton.py:374-378) */
 #define MUON_PREC_BF16_BSPLIT 1 /* B kept as a bf16 hi+lo pair, B*X accumulates both (needed for the constant-coefficient table) */
+#define MUON_PREC_F16 2         /* the iterate and both Gram-side matrices are kept in IEEE half inside the workspace (inputs
+                                   and the result stay bfloat16), each times a power of two that keeps it in the normal
+                                   range: eight times the mantissa of bfloat16 at the same matrix-core rate, no hi+lo pair
+                                   needed for any of the reference's coefficient tables */
 
 /* flags of muon_ns_batched */
 #define MUON_NS_CAST_INPUT_FIRST 1 /* fp32 input: round to bf16 BEFORE taking the norm (muon.py:883-888); default is

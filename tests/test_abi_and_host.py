@@ -230,4 +230,4 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             pending = set()
             continue
         assert not (regs(code) & pending), f"uses a transpose-read result before the wait: {line}"
-    assert kernels == 2 and reads >= 2 * 12 * 4
+    assert kernels == 4 and reads >= 4 * 12 * 4      # two tile configurations x {bfloat16, half} workspace

@@ -228,7 +228,7 @@ def test_config2_emerging_muon_full_step(gpu_device):
         opt.step()
     ev1.record()
     torch.cuda.synchronize()
-    print(f"config 2 emerging Muon: {ev0.elapsed_time(ev1) / 3:.1f} ms/step (msign 5 steps, hi+lo split on the last 3)", flush=True)
+    print(f"config 2 emerging Muon: {ev0.elapsed_time(ev1) / 3:.1f} ms/step (msign 5 steps, half-precision workspace)", flush=True)
 
 
 def test_scalar_groups_throughput(gpu_device):
