@@ -137,7 +137,11 @@ def newton_schulz(
              "bf16_gemm":   one bf16 rounding per GEMM epilogue, the rounding
                             points of newton_schulz_triton.py:374-378
              "bf16_gemm_bsplit": as bf16_gemm but B kept as a bf16 hi+lo pair
-    Returns bf16 for the bf16 modes and fp32 for "fp32", shaped like G.
+             "f16_gemm":    a model of the HIP path's half-precision workspace (no counterpart in the reference): one
+                            IEEE-half rounding per GEMM epilogue with X, A, B kept times 2^sx, 2^8, 2^6
+                            (sx = floor(log2 sqrt(m n)) - 3), a*I inside B after the first iteration where |a| <= 4.2,
+                            bf16 result
+    Returns bf16 for the bf16 / f16 modes and fp32 for "fp32", shaped like G.
     """
     if G.ndim < 2:
         raise ValueError("Newton-Schulz needs at least 2 dimensions")
@@ -173,6 +177,25 @@ def newton_schulz(
                     hi = _bf16_round(B)
                     lo = _bf16_round(B - hi)
                     X = _bf16_round(a * X + hi @ X + lo @ X)
+            X = X.to(torch.bfloat16)
+        elif storage == "f16_gemm":
+            m, n = X.shape[-2], X.shape[-1]
+            sx = max(int(math.floor(0.5 * math.log2(m * n))) - 3, 0)
+
+            def half(t: Tensor, shift: int) -> Tensor:
+                return (t * 2.0 ** shift).to(torch.float16).to(torch.float32) * 2.0 ** -shift
+
+            X = half(X, sx)
+            eye = torch.eye(m, dtype=torch.float32)
+            for it, (a, b, c) in enumerate(coeffs):
+                A = half(X @ X.mT, 8)
+                B = c * (A @ A) + b * A
+                last = it == len(coeffs) - 1
+                if it > 0 and abs(a) <= 4.2:
+                    Y = half(B + a * eye, 6) @ X
+                else:
+                    Y = a * X + half(B, 6) @ X
+                X = _bf16_round(Y) if last else half(Y, sx)
             X = X.to(torch.bfloat16)
         else:
             raise ValueError(f"unknown storage {storage!r}")

@@ -340,6 +340,10 @@ def test_half_precision_workspace(ns, gpu_device, shape, table):
     print("rel err", err, flush=True)
     assert err <= 4e-3
     assert err <= 0.5 * _rel(plain, want)
+    # the CPU model of the same rounding points (half storage, the same power-of-two factors, a*I inside B): what is
+    # left between the two is the order of the fp32 sums, which flips some of the final bf16 roundings
+    model = torch.stack([O.newton_schulz(x, coeffs, 1e-7, storage="f16_gemm", eps_mode=em) for x in mats]).reshape(G.shape)
+    assert _rel(got, model) <= 2.5e-3
 
 
 def test_half_precision_workspace_scales(ns, gpu_device):

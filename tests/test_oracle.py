@@ -95,6 +95,7 @@ def test_ns_eps_modes():
 @pytest.mark.parametrize("table,storage,bar", [
     ("quintic", "bf16_gemm", 1e-2), ("simple", "bf16_gemm_bsplit", 1e-2),
     ("quintic", "bf16_eager", 2e-2), ("simple", "bf16_eager", 4e-2),
+    ("quintic", "f16_gemm", 4e-3), ("simple", "f16_gemm", 4e-3), ("msign", "f16_gemm", 4e-3),
 ])
 def test_ns_bf16_modes_close_to_fp32(table, storage, bar):
     g = torch.Generator().manual_seed(5)
