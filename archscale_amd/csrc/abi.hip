@@ -78,15 +78,13 @@ size_t plan_bytes_bound(int batch, int rows, int cols, int prec_mode) {
 }
 
 int compute_units() {
-  static int n = 0;
-  if (n == 0) {
+  static const int n = [] {
     int dev = 0, v = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n = v;
-    else
-      n = 256;
-  }
+      return v;
+    return 256;
+  }();
   return n;
 }
 
