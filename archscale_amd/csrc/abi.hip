@@ -100,7 +100,7 @@ std::vector<ProfRec> g_prof;
 std::atomic<bool> g_prof_on{false};
 
 hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GroupedGemmParams& g, hipStream_t stream,
-                      double flops_algorithmic, double flops_issued, bool f16 = false) {
+                      double flops_algorithmic, double flops_issued, int f16 = 0) {
   if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16);
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   ProfRec r;
@@ -129,7 +129,7 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
 // is quartered as a whole up to QUARTER_MAX_ALONE tiles.  ARCHSCALE_MUON_QUARTER=0 switches it off.
 constexpr int QUARTER_MAX_TAIL = 128, QUARTER_MAX_ALONE = 176;
 hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp, hipStream_t stream,
-                         double fa, double fi, bool f16) {
+                         double fa, double fi, int f16) {
   static const bool enabled = !(getenv("ARCHSCALE_MUON_QUARTER") && atoi(getenv("ARCHSCALE_MUON_QUARTER")) == 0);
   const int total = gp.tile_start[gp.n_groups];
   const int round = 256;
@@ -339,24 +339,17 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     }
     e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);
     if (e != hipSuccess) return (int)e;
-    if (f16) {
-      // the unnormalised bfloat16 update cannot go into half as it is (its magnitude is the gradient's): one pass in
-      // place turns it into half(2^sx * X / |X|); the deferred scale of the bfloat16 path is then not used
-      e = launch_layout(P.Xt[0], MUON_DTYPE_BF16, 0, xs, pl.Mp, P.q.batch, pl.Np, pl.Mp, P.scale, P.Xt[0], xs, pl.Mp,
-                        pl.Np, pl.Mp, nullptr, 0, 0, stream, 1, P.sx);
-      if (e != hipSuccess) return (int)e;
-    }
   }
 
   // one product of the iteration for every problem: problems that share a tile configuration go into one
   // launch (at most MAX_GROUPS per launch)
-  auto run_mode = [&](int mode, bool last, auto&& fill) -> hipError_t {
+  auto run_mode = [&](int mode, bool last, int ws16, auto&& fill) -> hipError_t {
     for (int tile : {256, 128}) {
       GroupedGemmParams gp = {};
       double fa = 0.0, fi = 0.0;
       auto flush = [&]() -> hipError_t {
         if (gp.n_groups == 0) return hipSuccess;
-        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi, f16);
+        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi, ws16);
         gp = GroupedGemmParams{};
         fa = fi = 0.0;
         return err;
@@ -397,22 +390,31 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     // With the hi+lo pair the folded diagonal is exact; an iteration of a split call that keeps B in plain bf16 is not
     // folded (constant coefficients on small matrices: 8.4e-3 -> 1.1e-2 for 64x129 when it is).
     const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f && (!split_any || split);
+    // Half-precision workspace after the fused momentum: the unnormalised bfloat16 update cannot go into half as it is
+    // (its magnitude is the gradient's), so the first iteration runs on it in bfloat16 with the deferred scale, as in
+    // MUON_PREC_BF16, and its last product writes X' as scaled half.  The operand of that iteration is then the exact
+    // bfloat16 update, and A and B of ONE early iteration in bfloat16 cost nothing measurable (error against an fp32
+    // run, CPU model, 512x2048 / 1024x1024 / 64x129: constant row 2.15 / 2.01 / 2.27e-3 against 2.16 / 2.03 / 2.22e-3
+    // with all five iterations in half; a second bfloat16 iteration would cost 3.3 / 3.7 / 9.2e-3).
+    const bool lowp = f16 && fused && it == 0;
+    const int SAi = lowp ? 0 : SA, SBi = lowp ? 0 : SB;
+    const int ws16 = lowp ? 0 : (f16 ? 1 : 0);
     // A = X X^T, from X^T (K-major operand)
-    e = run_mode(MODE_SYRKT, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+    e = run_mode(MODE_SYRKT, last, ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
       g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
-      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, SA - 2 * P.sx); g.beta = 0.f;
-      g.scale = (fused && it == 0 && !f16) ? P.scale : nullptr;
+      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, SAi - 2 * (lowp ? 0 : P.sx)); g.beta = 0.f;
+      g.scale = (fused && it == 0) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
     });
     if (e != hipSuccess) return (int)e;
     // B = c A A + b A
-    e = run_mode(MODE_SYRK2, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+    e = run_mode(MODE_SYRK2, last, ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;
       const long as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
@@ -420,15 +422,15 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.E = P.A; g.strideE = as; g.lde = pl.Mp;
       g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp;
-      g.alpha = ldexpf(c, SB - 2 * SA); g.beta = ldexpf(b, SB - SA);
-      g.diag_add = fold ? ldexpf(a, SB) : 0.f;
+      g.alpha = ldexpf(c, SBi - 2 * SAi); g.beta = ldexpf(b, SBi - SAi);
+      g.diag_add = fold ? ldexpf(a, SBi) : 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
     });
     if (e != hipSuccess) return (int)e;
     // X' = a X + B X
-    e = run_mode(MODE_BX, last, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+    e = run_mode(MODE_BX, last, (lowp && !last) ? 2 : ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
@@ -436,9 +438,10 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.K = pl.Mp;
       g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
       g.E = fold ? nullptr : P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
-      g.alpha = ldexpf(a, SB); g.beta = 0.f;
-      g.out_shift = -SB - (last ? P.sx : 0);   // the caller's result is the iterate itself, without its factor
-      g.scale = (fused && it == 0 && !f16) ? P.scale : nullptr;
+      g.alpha = ldexpf(a, SBi); g.beta = 0.f;
+      // the operand carries 2^sx (not in the bfloat16 iteration), the next iterate does, the caller's result does not
+      g.out_shift = -SBi - (lowp ? 0 : P.sx) + ((last || !f16) ? 0 : P.sx);
+      g.scale = (fused && it == 0) ? P.scale : nullptr;
       if (!last) {
         g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {

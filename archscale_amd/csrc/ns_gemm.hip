@@ -60,12 +60,15 @@ __device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
 // 16-byte bank groups (rows alternate between the two 128-byte halves of the 64 banks).
 __device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * ROW_BYTES + ((c ^ ((r >> 1) & 7)) << 4); }
 
-// F16: the workspace matrices (operands, addend, non-final outputs) are IEEE half instead of bfloat16 (the caller's
+// F16 = 1: the workspace matrices (operands, addend, non-final outputs) are IEEE half instead of bfloat16 (the caller's
 // tensors stay bfloat16); the host keeps them in range with power-of-two factors folded into alpha / beta / out_shift.
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND, bool F16>
+// F16 = 2: bfloat16 operands and addend, IEEE-half output (the step from a bfloat16 iteration to a half one).
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND, int F16>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
 ns_gemm_kernel(const GroupedGemmParams gp) {
   static_assert(!(F16 && SPLIT), "the hi+lo pair is a bfloat16 device");
+  static_assert(F16 != 2 || (MODE == MODE_BX && !FINAL), "only X' changes its storage type");
+  constexpr bool IN16 = F16 == 1, OUT16 = F16 != 0;
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int WAVES_N = BN / WN;
   constexpr int FM = WM / 32, FN = WN / 32;
@@ -80,8 +83,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   // SPLIT means "B is a hi+lo pair": SYRK2 WRITES the pair, BX READS it as a second pass over K
   constexpr bool KSPLIT = SPLIT && MODE == MODE_BX;
   // element codecs: workspace data is half or bfloat16; the final launch writes the caller's bfloat16
-  auto dec = [](uint32_t bits) { return F16 ? f16_to_f32((uint16_t)bits) : bf16_to_f32((uint16_t)bits); };
-  auto enc = [](float f) { return (F16 && !FINAL) ? f16_bits(f) : bf16_bits(f); };
+  auto dec = [](uint32_t bits) { return IN16 ? f16_to_f32((uint16_t)bits) : bf16_to_f32((uint16_t)bits); };
+  auto enc = [](float f) { return (OUT16 && !FINAL) ? f16_bits(f) : bf16_bits(f); };
   auto pk4 = [&](float a, float b, float c, float d) {
     uint2 r;
     r.x = (uint32_t)enc(a) | ((uint32_t)enc(b) << 16);
@@ -276,7 +279,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 #pragma unroll
     for (int q = 0; q < NMF; ++q) {
       if (COMPUTE)
-        acc[q / FN][q % FN] = F16 ? __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[cbuf][q / FN]), __builtin_bit_cast(f16x8, bq[cbuf][q % FN]), acc[q / FN][q % FN], 0, 0, 0)
+        acc[q / FN][q % FN] = IN16 ? __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[cbuf][q / FN]), __builtin_bit_cast(f16x8, bq[cbuf][q % FN]), acc[q / FN][q % FN], 0, 0, 0)
                                   : __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cbuf][q / FN], bq[cbuf][q % FN], acc[q / FN][q % FN], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
       const int g_lo = g0 + (q * (g1 - g0) + NMF - 1) / NMF, g_hi = g0 + ((q + 1) * (g1 - g0) + NMF - 1) / NMF;
@@ -699,7 +702,7 @@ long ns_gemm_tiles(int mode, const GemmParams& p) {
   return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true, bool F16 = false>
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true, int F16 = 0>
 static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
@@ -722,40 +725,45 @@ static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN, bool F16>
+template <int BM, int BN, int WM, int WN, int F16>
 static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGemmParams& p, hipStream_t s) {
   if (F16 && split) return hipErrorInvalidValue;
-  switch (mode) {
-    case MODE_SYRK:
-      return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false, true, F16>(p, s);
-    case MODE_SYRKT:
-      return launch_one<BM, BN, WM, WN, MODE_SYRKT, false, false, true, F16>(p, s);
-    case MODE_SYRK2:
-      if constexpr (!F16) {
-        if (split) return launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s);
-      }
-      return launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false, true, F16>(p, s);
-    case MODE_BX:
-      if constexpr (!F16) {
-        if (split) {
-          if (p.g[0].E)
-            return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
-                          : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
-          return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true, false>(p, s)
-                        : launch_one<BM, BN, WM, WN, MODE_BX, true, false, false>(p, s);
+  if constexpr (F16 == 2) {
+    if (mode != MODE_BX || final_ || !p.g[0].E) return hipErrorInvalidValue;
+    return launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, 2>(p, s);
+  } else {
+    switch (mode) {
+      case MODE_SYRK:
+        return launch_one<BM, BN, WM, WN, MODE_SYRK, false, false, true, F16>(p, s);
+      case MODE_SYRKT:
+        return launch_one<BM, BN, WM, WN, MODE_SYRKT, false, false, true, F16>(p, s);
+      case MODE_SYRK2:
+        if constexpr (!F16) {
+          if (split) return launch_one<BM, BN, WM, WN, MODE_SYRK2, true, false>(p, s);
         }
-      }
-      if (p.g[0].E)
-        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, true, F16>(p, s)
-                      : launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, F16>(p, s);
-      return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, false, F16>(p, s)
-                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false, F16>(p, s);
+        return launch_one<BM, BN, WM, WN, MODE_SYRK2, false, false, true, F16>(p, s);
+      case MODE_BX:
+        if constexpr (!F16) {
+          if (split) {
+            if (p.g[0].E)
+              return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true>(p, s)
+                            : launch_one<BM, BN, WM, WN, MODE_BX, true, false>(p, s);
+            return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, true, true, false>(p, s)
+                          : launch_one<BM, BN, WM, WN, MODE_BX, true, false, false>(p, s);
+          }
+        }
+        if (p.g[0].E)
+          return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, true, F16>(p, s)
+                        : launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, F16>(p, s);
+        return final_ ? launch_one<BM, BN, WM, WN, MODE_BX, false, true, false, F16>(p, s)
+                      : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false, F16>(p, s);
+    }
+    return hipErrorInvalidValue;
   }
-  return hipErrorInvalidValue;
 }
 
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
-                                  hipStream_t stream, bool f16) {
+                                  hipStream_t stream, int f16) {
   if (gp.n_groups < 1 || gp.n_groups > MAX_GROUPS) return hipErrorInvalidValue;
   const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2 || mode == MODE_SYRKT);
   for (int i = 0; i < gp.n_groups; ++i) {
@@ -774,13 +782,16 @@ hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, c
       if (g.qt_first + blocks / 4 > coarse) return hipErrorInvalidValue;
     }
   }
-  if (f16) {
-    if (tile == 256) return launch_cfg<256, 256, 128, 64, true>(mode, split, final_, gp, stream);
-    if (tile == 128) return launch_cfg<128, 128, 64, 64, true>(mode, split, final_, gp, stream);
-    return hipErrorInvalidValue;
+  if (f16 == 1) {
+    if (tile == 256) return launch_cfg<256, 256, 128, 64, 1>(mode, split, final_, gp, stream);
+    if (tile == 128) return launch_cfg<128, 128, 64, 64, 1>(mode, split, final_, gp, stream);
+  } else if (f16 == 2) {
+    if (tile == 256) return launch_cfg<256, 256, 128, 64, 2>(mode, split, final_, gp, stream);
+    if (tile == 128) return launch_cfg<128, 128, 64, 64, 2>(mode, split, final_, gp, stream);
+  } else if (f16 == 0) {
+    if (tile == 256) return launch_cfg<256, 256, 128, 64, 0>(mode, split, final_, gp, stream);
+    if (tile == 128) return launch_cfg<128, 128, 64, 64, 0>(mode, split, final_, gp, stream);
   }
-  if (tile == 256) return launch_cfg<256, 256, 128, 64, false>(mode, split, final_, gp, stream);
-  if (tile == 128) return launch_cfg<128, 128, 64, 64, false>(mode, split, final_, gp, stream);
   return hipErrorInvalidValue;
 }
 

@@ -36,7 +36,8 @@ extern "C" {
 #define MUON_PREC_F16 2         /* the iterate and both Gram-side matrices are kept in IEEE half inside the workspace (inputs
                                    and the result stay bfloat16), each times a power of two that keeps it in the normal
                                    range: eight times the mantissa of bfloat16 at the same matrix-core rate, no hi+lo pair
-                                   needed for any of the reference's coefficient tables */
+                                   needed for any of the reference's coefficient tables (muon_momentum_ns_grouped runs the
+                                   first iteration in bfloat16 on the unnormalised update and goes to half from there) */
 
 /* flags of muon_ns_batched */
 #define MUON_NS_CAST_INPUT_FIRST 1 /* fp32 input: round to bf16 BEFORE taking the norm (muon.py:883-888); default is

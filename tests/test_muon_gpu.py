@@ -413,6 +413,38 @@ def test_emerging_fused_momentum_matches_separate_calls(gpu_device, nesterov):
         assert _rel(a, b) <= 3e-3
 
 
+@pytest.mark.parametrize("table", ["quintic", "simple", "one_row"])
+def test_fused_momentum_with_half_precision_workspace(gpu_device, table):
+    """``ns_precision="f16"`` on the fused path: the first iteration runs in bfloat16 on the unnormalised update (deferred
+    scale) and hands the iterate over as scaled half.  From zero momentum with Nesterov the update is (1 + mu) G, and with
+    fp32 weights, no weight decay and no lr adjustment the orthogonalised update is (W0 - W1) / lr: it must stay within
+    the half-precision bar of an fp32 run, well below what bfloat16 storage gives, and agree with the unfused path."""
+    from archscale_amd.optim.muon import Muon
+    shapes = [(512, 768), (768, 512), (2, 256, 640), (96, 200), (320, 129)]   # 256- and 128-tile classes, ragged, 3-D
+    coeffs = {"quintic": O.QUINTIC, "simple": list(O.SIMPLE) * 5, "one_row": list(O.SIMPLE)}[table]
+    grads = _grads(shapes, torch.float32, 41)
+    mu, lr = 0.9, 0.5
+    want = [O.newton_schulz(((1.0 + mu) * g).to(torch.bfloat16), coeffs, 1e-8, storage="fp32").float() for g in grads]
+    got = {}
+    for prec, fuse in (("f16", True), ("f16", False), ("bf16", True)):
+        params = _make(shapes, torch.float32, 12, gpu_device)
+        w0 = [p.detach().clone() for p in params]
+        opt = Muon(params, lr=lr, mu=mu, weight_decay=0.0, epsilon=1e-8, nesterov=True, adjust_lr=None,
+                   ns_coefficients=coeffs, ns_precision=prec, fuse_momentum=fuse)
+        for p, g in zip(params, grads):
+            p.grad = g.to(gpu_device)
+        opt.step()
+        torch.cuda.synchronize()
+        got[(prec, fuse)] = [((w - p.detach()) / lr).cpu() for w, p in zip(w0, params)]
+    for i, w in enumerate(want):
+        e16, e16u, ebf = (_rel(got[k][i], w) for k in (("f16", True), ("f16", False), ("bf16", True)))
+        print(table, shapes[i], "f16 fused %.2e  f16 unfused %.2e  bf16 fused %.2e" % (e16, e16u, ebf), flush=True)
+        assert e16 <= 4e-3 and e16u <= 4e-3
+        if table != "one_row":
+            assert e16 <= 0.6 * ebf
+        assert _rel(got[("f16", True)][i], got[("f16", False)][i]) <= 3e-3
+
+
 def test_random_parameter_sets(gpu_device):
     """Seeded sweep: parameter sets with ragged 2-D and 3-D shapes, both weight dtypes, plain and MuonH updates, with and
     without Nesterov, weight decay and the fused momentum path; two steps each against the reference-semantics oracle
