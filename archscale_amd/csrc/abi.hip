@@ -565,7 +565,7 @@ int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_
 namespace {
 struct SnPlan {
   NsPlan pl;
-  size_t off_x, off_g, off_z, off_part, total;
+  size_t off_x, off_g, off_g2, off_g4, off_xscale, off_xpart, off_z, off_part, total;
 };
 SnPlan make_sn_plan(int batch, int rows, int cols) {
   SnPlan s;
@@ -574,6 +574,10 @@ SnPlan make_sn_plan(int batch, int rows, int cols) {
   auto take = [&](size_t bytes) { size_t o = off; off = (size_t)round_up((long)(off + bytes), 256); return o; };
   s.off_x = take((size_t)batch * s.pl.Mp * s.pl.Np * 2);
   s.off_g = take((size_t)batch * s.pl.Mp * s.pl.Mp * 2);
+  s.off_g2 = take((size_t)batch * s.pl.Mp * s.pl.Mp * 2);   // G^2 and G^4 of the grouped rounds (used from 6 / 16 rounds on)
+  s.off_g4 = take((size_t)batch * s.pl.Mp * s.pl.Mp * 2);
+  s.off_xscale = take((size_t)batch * sizeof(float));
+  s.off_xpart = take((size_t)batch * (s.pl.Mp / 64) * (s.pl.Np / 64) * sizeof(float));
   s.off_z = take((size_t)2 * batch * s.pl.Mp * sizeof(float));
   s.off_part = take((size_t)2 * batch * (s.pl.Mp / SN_ROWS) * 2 * sizeof(float));
   s.total = off;
@@ -608,7 +612,8 @@ int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   // tall: the matrix meant (after MUON_SN_TRANSPOSED) has more rows than columns; use_t: its short-side-first copy is
   // the transpose of the stored block
-  struct Prob { muon_sn_problem q; SnPlan sp; __bf16 *X, *G; float *z, *part; bool tall, use_t; };
+  struct Prob { muon_sn_problem q; SnPlan sp; __bf16 *X, *G, *G2, *G4; float *xscale, *xpart, *z, *part; bool tall, use_t; };
+  const int levels = spectral_power_levels(steps);
   std::vector<Prob> pr(n_problems);
   size_t off = 0;
   for (int i = 0; i < n_problems; ++i) {
@@ -623,6 +628,10 @@ int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int
     off += P.sp.total;
     P.X = (__bf16*)(ws + P.sp.off_x);
     P.G = (__bf16*)(ws + P.sp.off_g);
+    P.G2 = levels >= 1 ? (__bf16*)(ws + P.sp.off_g2) : nullptr;
+    P.G4 = levels >= 2 ? (__bf16*)(ws + P.sp.off_g4) : nullptr;
+    P.xscale = (float*)(ws + P.sp.off_xscale);
+    P.xpart = (float*)(ws + P.sp.off_xpart);
     P.z = (float*)(ws + P.sp.off_z);
     P.part = (float*)(ws + P.sp.off_part);
     const bool transposed = (P.q.flags & MUON_SN_TRANSPOSED) != 0;
@@ -630,73 +639,98 @@ int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int
     P.use_t = transposed != P.tall;
   }
   hipError_t e;
-  // bf16 copy of every matrix with its short side first, zero padded to the GEMM tile
+  // bf16 copy of every matrix with its short side first, zero padded to the GEMM tile, and its sums of squares per tile
   for (const Prob& P : pr) {
     const NsPlan& pl = P.sp.pl;
     const long xs = (long)pl.Mp * pl.Np;
+    const size_t xt = (size_t)(pl.Mp / 64) * (pl.Np / 64);
     for (int b = 0; b < P.q.batch; ++b) {
       if (!P.use_t)
         e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, P.X + b * xs, xs,
-                          pl.Np, pl.Mp, pl.Np, nullptr, 0, 0, stream);
+                          pl.Np, pl.Mp, pl.Np, nullptr, 0, 0, stream, 0, 0, P.xpart + b * xt);
       else
         e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, nullptr, 0, 0,
-                          pl.Np, pl.Mp, P.X + b * xs, xs, pl.Np, stream);
+                          pl.Np, pl.Mp, P.X + b * xs, xs, pl.Np, stream, 0, 0, P.xpart + b * xt);
       if (e != hipSuccess) return (int)e;
     }
   }
-  // G = X X^T: problems of one tile size share launches
-  for (int tile : {256, 128}) {
-    GroupedGemmParams gp = {};
-    auto flush = [&]() -> hipError_t {
-      if (gp.n_groups == 0) return hipSuccess;
-      hipError_t err = launch_ns_gemm_grouped(tile, MODE_SYRK, false, false, gp, stream);
-      gp = GroupedGemmParams{};
-      return err;
-    };
-    for (const Prob& P : pr) {
-      const NsPlan& pl = P.sp.pl;
-      if (pl.tile != tile) continue;
-      GemmParams g = {};
-      g.batch = P.q.batch;
-      g.P = P.X; g.Q = P.X; g.strideP = g.strideQ = (long)pl.Mp * pl.Np; g.ldp = g.ldq = pl.Np; g.K = pl.Np;
-      g.tilesM = g.tilesN = pl.Mp / pl.tile;
-      g.C = P.G; g.strideC = (long)pl.Mp * pl.Mp; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
-      const long tiles = ns_gemm_tiles(MODE_SYRK, g);
-      if (tiles > 0x7ffffff0L) return MUON_E_UNSUPPORTED;
-      if (gp.n_groups == MAX_GROUPS || tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L) {
-        if ((e = flush()) != hipSuccess) return (int)e;
+  // a symmetric product for every problem, problems of one tile size sharing launches: dst = scale^2 * src src^T
+  // (src: [d_p][K] row-major per matrix)
+  auto gram = [&](auto&& src_of, auto&& k_of, auto&& dst_of, auto&& scale_of) -> int {
+    for (int tile : {256, 128}) {
+      GroupedGemmParams gp = {};
+      auto flush = [&]() -> hipError_t {
+        if (gp.n_groups == 0) return hipSuccess;
+        hipError_t err = launch_ns_gemm_grouped(tile, MODE_SYRK, false, false, gp, stream);
+        gp = GroupedGemmParams{};
+        return err;
+      };
+      for (const Prob& P : pr) {
+        const NsPlan& pl = P.sp.pl;
+        if (pl.tile != tile) continue;
+        GemmParams g = {};
+        const int K = k_of(P);
+        g.batch = P.q.batch;
+        g.P = src_of(P); g.Q = g.P; g.strideP = g.strideQ = (long)pl.Mp * K; g.ldp = g.ldq = K; g.K = K;
+        g.tilesM = g.tilesN = pl.Mp / pl.tile;
+        g.C = dst_of(P); g.strideC = (long)pl.Mp * pl.Mp; g.ldc = pl.Mp; g.alpha = 1.f; g.beta = 0.f;
+        g.scale = scale_of(P);
+        const long tiles = ns_gemm_tiles(MODE_SYRK, g);
+        if (tiles > 0x7ffffff0L) return MUON_E_UNSUPPORTED;
+        if (gp.n_groups == MAX_GROUPS || tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L) {
+          if ((e = flush()) != hipSuccess) return (int)e;
+        }
+        gp.g[gp.n_groups] = g;
+        gp.tile_start[gp.n_groups + 1] = gp.tile_start[gp.n_groups] + (int)tiles;
+        ++gp.n_groups;
       }
-      gp.g[gp.n_groups] = g;
-      gp.tile_start[gp.n_groups + 1] = gp.tile_start[gp.n_groups] + (int)tiles;
-      ++gp.n_groups;
+      if ((e = flush()) != hipSuccess) return (int)e;
     }
-    if ((e = flush()) != hipSuccess) return (int)e;
-  }
-  // the rounds: classes of one orientation share a launch sequence
-  for (int kind = 0; kind < 2; ++kind) {
+    return 0;
+  };
+  // the classes in launches of at most SN_MAX_CLASSES
+  auto for_class_chunks = [&](auto&& run) -> int {
     SnParams sp = {};
-    auto flush = [&]() -> hipError_t {
-      if (sp.n == 0) return hipSuccess;
-      hipError_t err = launch_spectral_iterate(sp, steps, stream);
-      sp = SnParams{};
-      return err;
-    };
-    for (const Prob& P : pr) {
-      if ((int)P.tall != kind) continue;
+    for (size_t i = 0; i <= pr.size(); ++i) {
+      if (i == pr.size() || sp.n == SN_MAX_CLASSES ||
+          (long)pr[i].q.batch * (pr[i].sp.pl.Mp / SN_ROWS) + sp.blk_start[sp.n] > 0x3ffffff0L) {
+        if (sp.n > 0 && (e = run(sp)) != hipSuccess) return (int)e;
+        sp = SnParams{};
+        if (i == pr.size()) break;
+      }
+      const Prob& P = pr[i];
       const NsPlan& pl = P.sp.pl;
       const long blocks = (long)P.q.batch * (pl.Mp / SN_ROWS);
       if (blocks > 0x3ffffff0L) return MUON_E_UNSUPPORTED;
-      if (sp.n == SN_MAX_CLASSES || blocks + sp.blk_start[sp.n] > 0x3ffffff0L) {
-        if ((e = flush()) != hipSuccess) return (int)e;
-      }
       SnClass& c = sp.c[sp.n];
-      c.X = P.X; c.G = P.G; c.z = P.z; c.part = P.part; c.sigma = P.q.sigma_out;
+      c.X = P.X; c.G = P.G; c.G2 = P.G2; c.G4 = P.G4;
+      c.xscale = P.xscale; c.xpart = P.xpart; c.xtiles = (pl.Mp / 64) * (pl.Np / 64);
+      c.z = P.z; c.part = P.part; c.sigma = P.q.sigma_out;
       c.batch = P.q.batch; c.d = pl.m; c.d_p = pl.Mp; c.L_p = pl.Np; c.nblk = pl.Mp / SN_ROWS; c.tall = P.tall ? 1 : 0;
       sp.blk_start[sp.n + 1] = sp.blk_start[sp.n] + (int)blocks;
       ++sp.n;
     }
-    if ((e = flush()) != hipSuccess) return (int)e;
+    return 0;
+  };
+  int st;
+  // G = s^2 X X^T with s a power of two near sqrt(d) / |X|_F (mean eigenvalue about 1: no power of G leaves the bf16 range)
+  if ((st = for_class_chunks([&](const SnParams& sp) { return launch_spectral_xscale(sp, stream); })) != 0) return st;
+  if ((st = gram([](const Prob& P) { return P.X; }, [](const Prob& P) { return P.sp.pl.Np; },
+                 [](const Prob& P) { return P.G; }, [](const Prob& P) { return (const float*)P.xscale; })) != 0)
+    return st;
+  // G2 = G^2, G4 = G2^2
+  if (levels >= 1) {
+    if ((st = gram([](const Prob& P) { return P.G; }, [](const Prob& P) { return P.sp.pl.Mp; },
+                   [](const Prob& P) { return P.G2; }, [](const Prob&) { return (const float*)nullptr; })) != 0)
+      return st;
   }
+  if (levels >= 2) {
+    if ((st = gram([](const Prob& P) { return P.G2; }, [](const Prob& P) { return P.sp.pl.Mp; },
+                   [](const Prob& P) { return P.G4; }, [](const Prob&) { return (const float*)nullptr; })) != 0)
+      return st;
+  }
+  // the rounds: every application of G (or of a power of it) is one launch over all classes
+  if ((st = for_class_chunks([&](const SnParams& sp) { return launch_spectral_iterate(sp, steps, stream); })) != 0) return st;
   return 0;
 }
 

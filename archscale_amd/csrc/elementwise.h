@@ -37,10 +37,12 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
                              hipStream_t stream);
 
 // D = bf16(scale*in) in the input's orientation and T = its transpose (either may be null), both zero-padded to
-// d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).
+// d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).  tile_sumsq (optional): the sum of
+// squares of the values written, one float per 64x64 tile: [batch][d_rows / 64][d_cols / 64].
 hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
-                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16 = 0, int out_shift = 0);
+                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16 = 0, int out_shift = 0,
+                         float* tile_sumsq = nullptr);
 
 // momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
 constexpr int MOMLAY_MAX = 32;

@@ -237,9 +237,12 @@ __global__ void __launch_bounds__(256)
 normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, int cols, int ld,
                         const float* __restrict__ scale,
                         uint16_t* __restrict__ D, long d_bstride, int ldd, int d_rows, int d_cols,
-                        uint16_t* __restrict__ T, long t_bstride, int ldt, int out_f16, int out_shift) {
+                        uint16_t* __restrict__ T, long t_bstride, int ldt, int out_f16, int out_shift,
+                        float* __restrict__ tile_sumsq) {
   // 64x64 tile; d_rows/d_cols are the padded extents (multiples of 64)
   __shared__ uint16_t tile[64][66];
+  __shared__ float red[4];
+  float ss[1] = {0.f};
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const char* base = (const char*)in + (size_t)b * in_bstride * sizeof(typename Elem<DT>::T);
@@ -265,6 +268,7 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
       // half output: times 2^out_shift, which keeps the normalised entries in the normal range of the format
       o[k] = out_f16 ? __builtin_bit_cast(uint16_t, (_Float16)(x * s * fs)) : f2bf(x * s);
       tile[tr + h * 32][tc + k] = o[k];
+      if (tile_sumsq) { const float w = out_f16 ? x * s : bf2f(o[k]); ss[0] += w * w; }
     }
     if (D && r < d_rows && c < d_cols) {
       uint4 pk;
@@ -272,6 +276,11 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
       pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
       *(uint4*)(D + (size_t)b * d_bstride + (size_t)r * ldd + c) = pk;
     }
+  }
+  if (tile_sumsq) {   // sum of squares of what this block wrote (every block of the grid: one value per 64x64 tile)
+    block_reduce<1>(ss, red);
+    if (threadIdx.x == 0)
+      tile_sumsq[((size_t)b * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x] = ss[0];
   }
   if (!T) return;
   __syncthreads();
@@ -312,13 +321,14 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
 
 hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
                          int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
-                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16, int out_shift) {
+                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16, int out_shift,
+                         float* tile_sumsq) {
   if (batch > 65535 || d_rows / 64 > 65535 || d_rows % 64 || d_cols % 64) return hipErrorInvalidValue;
   dim3 g3(d_cols / 64, d_rows / 64, batch);
 #define ARCHSCALE_NL(DT, CF)                                                                                   \
   hipLaunchKernelGGL((normalize_layout_kernel<DT, CF>), g3, dim3(256), 0, stream, in, in_bstride, rows, cols,  \
                      ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride, ldt,    \
-                     out_f16, out_shift)
+                     out_f16, out_shift, tile_sumsq)
   if (in_dtype == DT_BF16) ARCHSCALE_NL(DT_BF16, false);
   else if (cast_first) ARCHSCALE_NL(DT_F32, true);
   else ARCHSCALE_NL(DT_F32, false);

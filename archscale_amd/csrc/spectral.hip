@@ -9,8 +9,13 @@
 //   rows >  cols:  G = W^T W,  x0 = 1,      x = G^steps x0,        sigma^2 = x^T G x / x^T x
 //   rows <= cols:  G = W W^T,  x0 = W 1,    x = G^(steps-1) x0,    sigma^2 = |G x|^2 / x^T G x
 // which is the same vector sequence ((W^T W)^k 1 = W^T (W W^T)^(k-1) W 1) at 1/2 .. 1/11 of the memory
-// traffic per round.  Vectors stay in fp32 (the reference rounds them to bf16 every round); every round
-// is ONE launch over all matrices of all shape classes; norms are ordered two-stage reductions.
+// traffic per round.  The normalisation between two rounds only scales the vector, so all applications but the last
+// (whose Rayleigh quotient is the result, and is taken with G itself) may be grouped: with G2 = G^2 and G4 = G2^2,
+// formed once by the same SYRK kernel, 50 rounds are 12 passes over G4, one over G2 or G and the final one over G
+// instead of 50 or 51 passes over G.  G carries a power-of-two factor (mean eigenvalue about 1) that keeps its powers
+// in the bf16 range; the result is divided by it.  A rounding error in G2 / G4 perturbs the direction only, and the quotient is
+// second-order in it.  Vectors stay in fp32 (the reference rounds them to bf16 every round); every application is ONE
+// launch over all matrices of all shape classes; norms are ordered two-stage reductions.
 //
 // The weight update fuses decoupled weight decay, retraction to the spectral sphere and the step:
 //   W <- f * decay * W - lr * ratio * Phi,   f from sigma(decay * W) = decay * sigma(W)
@@ -118,13 +123,18 @@ sn_init_kernel(const SnParams sp) {
   }
 }
 
-// z[dst] <- G z[src] / max(|z[src]|, 1e-12);  part[dst] <- per strip (|z[dst]|^2,  z[src]^T z[dst] / |z[src]|)
+// z[dst] <- M z[src] / max(|z[src]|, 1e-12);  part[dst] <- per strip (|z[dst]|^2,  z[src]^T z[dst] / |z[src]|)
+// M = G, G2 or G4 (which = 0, 1, 2) and the source buffer are given per kind of class (wide, tall), whose sequences
+// differ; which < 0: the classes of that kind sit this launch out.
 __global__ void __launch_bounds__(256)
-sn_step_kernel(const SnParams sp, int src) {
+sn_step_kernel(const SnParams sp, int src_wide, int which_wide, int src_tall, int which_tall) {
   __shared__ float red[8];
   int g, b, s;
   if (!locate(sp, g, b, s)) return;
   const SnClass c = sp.c[g];
+  const int src = c.tall ? src_tall : src_wide, which = c.tall ? which_tall : which_wide;
+  if (which < 0) return;
+  const __bf16* M = which == 0 ? c.G : (which == 1 ? c.G2 : c.G4);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int dst = src ^ 1;
   const float* zin = c.z + ((size_t)src * c.batch + b) * c.d_p;
@@ -135,7 +145,7 @@ sn_step_kernel(const SnParams sp, int src) {
   const float inv = 1.f / fmaxf(sqrtf(Sin), 1e-12f);
   const int r0 = s * SN_ROWS + wave * 4;
   float acc[4];
-  rows4_dot((const uint16_t*)c.G + (size_t)b * c.d_p * c.d_p + (size_t)r0 * c.d_p, c.d_p, zin, c.d_p, lane, acc);
+  rows4_dot((const uint16_t*)M + (size_t)b * c.d_p * c.d_p + (size_t)r0 * c.d_p, c.d_p, zin, c.d_p, lane, acc);
   float S = 0.f, D = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -155,42 +165,95 @@ sn_step_kernel(const SnParams sp, int src) {
 
 // sigma[b] from the partials of the last round
 __global__ void __launch_bounds__(64)
-sn_final_kernel(const SnParams sp, int src) {
+sn_final_kernel(const SnParams sp, int src_wide, int src_tall) {
   // one wave per matrix: blocks are numbered class by class
   int blk = blockIdx.x, g = 0;
   while (g < sp.n && blk >= sp.c[g].batch) { blk -= sp.c[g].batch; ++g; }
   if (g >= sp.n) return;
   const SnClass c = sp.c[g];
+  const int src = c.tall ? src_tall : src_wide;
   const int lane = threadIdx.x;
   float S, D;
   sum_pairs(c.part + (((size_t)src * c.batch + blk) * c.nblk) * 2, c.nblk, lane, S, D);
   const float s2 = c.tall ? D : (D > 0.f ? S / D : 0.f);
-  if (lane == 0) c.sigma[blk] = sqrtf(fmaxf(s2, 0.f));
+  const float xs = c.xscale[blk];   // G = xs^2 X X^T
+  if (lane == 0) c.sigma[blk] = xs > 0.f ? sqrtf(fmaxf(s2, 0.f)) / xs : 0.f;
+}
+
+// xscale[b]: one wave per matrix, blocks numbered class by class; the tile sums are added in a fixed order
+__global__ void __launch_bounds__(64)
+sn_xscale_kernel(const SnParams sp) {
+  int blk = blockIdx.x, g = 0;
+  while (g < sp.n && blk >= sp.c[g].batch) { blk -= sp.c[g].batch; ++g; }
+  if (g >= sp.n) return;
+  const SnClass c = sp.c[g];
+  const float* part = c.xpart + (size_t)blk * c.xtiles;
+  float t = 0.f;
+  for (int i = threadIdx.x; i < c.xtiles; i += 64) t += part[i];
+  t = wave_sum(t);
+  // a power of two: X and G are scaled exactly
+  if (threadIdx.x == 0) c.xscale[blk] = t > 0.f ? exp2f(rintf(0.5f * log2f((float)c.d / t))) : 0.f;
+}
+
+int spectral_power_levels(int steps) {
+  // G^4 pays from about a dozen applications on (two symmetric products against 3/4 of the passes), G^2 from half of that
+  return steps >= 16 ? 2 : (steps >= 6 ? 1 : 0);
+}
+
+hipError_t launch_spectral_xscale(const SnParams& sp, hipStream_t stream) {
+  if (sp.n < 1 || sp.n > SN_MAX_CLASSES) return hipErrorInvalidValue;
+  int matrices = 0;
+  for (int g = 0; g < sp.n; ++g) {
+    if (sp.c[g].batch <= 0 || !sp.c[g].xscale || !sp.c[g].xpart || sp.c[g].xtiles < 1) return hipErrorInvalidValue;
+    matrices += sp.c[g].batch;
+  }
+  hipLaunchKernelGGL(sn_xscale_kernel, dim3(matrices), dim3(64), 0, stream, sp);
+  return hipGetLastError();
 }
 
 hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t stream) {
   if (sp.n < 1 || sp.n > SN_MAX_CLASSES || steps < 1) return hipErrorInvalidValue;
   const int blocks = sp.blk_start[sp.n];
-  int matrices = 0, rounds = 0;
+  int matrices = 0;
+  bool have2 = true, have4 = true, any[2] = {false, false};
   for (int g = 0; g < sp.n; ++g) {
     const SnClass& c = sp.c[g];
-    if (c.batch <= 0 || c.d <= 0 || c.d_p % 128 || c.L_p % 8 || c.d > c.d_p || c.nblk * SN_ROWS != c.d_p) return hipErrorInvalidValue;
+    if (c.batch <= 0 || c.d <= 0 || c.d_p % 128 || c.L_p % 8 || c.d > c.d_p || c.nblk * SN_ROWS != c.d_p || !c.xscale)
+      return hipErrorInvalidValue;
     matrices += c.batch;
+    have2 = have2 && c.G2 != nullptr;
+    have4 = have4 && c.G4 != nullptr;
+    any[c.tall ? 1 : 0] = true;
   }
   if (blocks <= 0) return hipErrorInvalidValue;
   hipLaunchKernelGGL(sn_init_kernel, dim3(blocks), dim3(256), 0, stream, sp);
-  // a class whose matrices are tall needs one more application than one whose matrices are wide; both kinds can
-  // share a launch sequence only if they agree, so the caller passes classes of ONE kind per call
-  const bool tall = sp.c[0].tall != 0;
-  for (int g = 1; g < sp.n; ++g)
-    if ((sp.c[g].tall != 0) != tall) return hipErrorInvalidValue;
-  rounds = tall ? steps + 1 : steps;
-  int src = 0;
-  for (int r = 0; r < rounds; ++r) {
-    hipLaunchKernelGGL(sn_step_kernel, dim3(blocks), dim3(256), 0, stream, sp, src);
-    src ^= 1;
+  // applications before the final one: `steps` for tall matrices (one more than for wide ones, see the file comment),
+  // as many as possible with the highest power
+  int seq[2][3];   // per kind: how many applications of G4, G2, G, in this order
+  int len[2];
+  for (int kind = 0; kind < 2; ++kind) {
+    int n = kind ? steps : steps - 1;
+    seq[kind][0] = have4 ? n / 4 : 0; n -= 4 * seq[kind][0];
+    seq[kind][1] = have2 ? n / 2 : 0; n -= 2 * seq[kind][1];
+    seq[kind][2] = n;
+    len[kind] = any[kind] ? seq[kind][0] + seq[kind][1] + seq[kind][2] : 0;
   }
-  hipLaunchKernelGGL(sn_final_kernel, dim3(matrices), dim3(64), 0, stream, sp, src);
+  auto which_at = [&](int kind, int i) {   // matrix of application i of a kind; -1 past its end
+    if (i >= len[kind]) return -1;
+    if (i < seq[kind][0]) return 2;
+    if (i < seq[kind][0] + seq[kind][1]) return 1;
+    return 0;
+  };
+  int src[2] = {0, 0};
+  const int launches = len[0] > len[1] ? len[0] : len[1];
+  for (int i = 0; i <= launches; ++i) {
+    // the last launch is the final application of G for both kinds
+    const int w0 = i == launches ? (any[0] ? 0 : -1) : which_at(0, i), w1 = i == launches ? (any[1] ? 0 : -1) : which_at(1, i);
+    hipLaunchKernelGGL(sn_step_kernel, dim3(blocks), dim3(256), 0, stream, sp, src[0], w0, src[1], w1);
+    if (w0 >= 0) src[0] ^= 1;
+    if (w1 >= 0) src[1] ^= 1;
+  }
+  hipLaunchKernelGGL(sn_final_kernel, dim3(matrices), dim3(64), 0, stream, sp, src[0], src[1]);
   return hipGetLastError();
 }
 

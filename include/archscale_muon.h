@@ -238,7 +238,9 @@ int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_
  * muon_spectral_norm estimates the top singular value of every matrix of every shape class with the vector
  * sequence of power_iteration (emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:151-166:
  * v <- normalize(W^T (W v)) `steps` times from v = 1, sigma = |W v|), run on the Gram matrix of the short side
- * (one SYRK on the matrix cores per call, then one launch per round over all matrices; fp32 vectors).
+ * (one SYRK on the matrix cores per call, then launches over all matrices with fp32 vectors; from 6 / 16 rounds on the
+ * Gram matrix is squared once / twice, so that one pass stands for two / four rounds: the normalisation between
+ * rounds only scales the vector; the last application, whose quotient is the result, is always the Gram matrix's).
  * A problem is one shape class: `batch` matrices rows x cols with leading dimension ld, given by a HOST array of
  * device pointers (the parameters of a model are separate allocations); the matrix is read as bf16 (fp32 input is
  * rounded first, as the reference does, :158).  sigma_out: device, `batch` floats per problem.

@@ -22,7 +22,7 @@ def _rel(a, b):
 
 
 @pytest.mark.parametrize("shape", [(48, 160), (160, 48), (64, 64), (300, 700), (700, 300), (512, 2048), (2048, 512), (1, 40), (40, 1)])
-@pytest.mark.parametrize("steps", [1, 2, 7, 50])
+@pytest.mark.parametrize("steps", [1, 2, 6, 7, 16, 19, 50])
 def test_spectral_norm_matches_the_definition(gpu_device, shape, steps):
     from archscale_amd.emerging.spectral_ball_utils import spectral_norm
     g = torch.Generator().manual_seed(shape[0] * 7 + shape[1] + steps)
@@ -32,6 +32,20 @@ def test_spectral_norm_matches_the_definition(gpu_device, shape, steps):
     assert abs(got - want) / want < SIGMA_TOL, (got, want)
     ref = float(B.power_iteration(W, steps)[0])
     assert abs(got - ref) / ref < SIGMA_REF_TOL
+
+
+@pytest.mark.parametrize("shape", [(96, 200), (200, 96), (256, 256)])
+def test_spectral_norm_scales_with_the_matrix(gpu_device, shape):
+    """The grouped rounds run on powers of the Gram matrix that the library rescales by its trace: a matrix times a
+    power of two (exact in bf16) must give exactly that multiple of sigma, up to fp32 rounding, from 2^-30 to 2^20."""
+    from archscale_amd.emerging.spectral_ball_utils import spectral_norm
+    g = torch.Generator().manual_seed(shape[0] + 3 * shape[1])
+    W = (torch.randn(*shape, generator=g) * 0.02).to(torch.bfloat16)
+    base = spectral_norm(W.to(gpu_device), 50).item()
+    assert abs(base - B.power_iteration_fp64(W, 50)) < SIGMA_TOL * base
+    for e in (-30, -12, 9, 20):
+        got = spectral_norm((W.float() * 2.0 ** e).to(torch.bfloat16).to(gpu_device), 50).item()
+        assert abs(got / 2.0 ** e - base) <= 1e-4 * base, (e, got / 2.0 ** e, base)
 
 
 def test_spectral_norm_batches_dtypes_strides_and_zero(gpu_device):
