@@ -6,8 +6,8 @@ Per step and matrix the reference runs, in a Python loop over parameters and ove
 sigma, an in-place retraction, msign of the momentum and the update.  Here a param group is
 
   1 multi-tensor launch   momentum (+ l2 decay) of every parameter,
-  1 call                  spectral norms of every piece of every parameter (Gram matrices on the matrix cores, then one
-                          launch per round over all pieces; no host read),
+  1 call                  spectral norms of every piece of every parameter (Gram matrices and their 2nd / 4th powers on the
+                          matrix cores, then one launch per four rounds over all pieces; no host read),
   1 grouped call          msign of every piece (strided views into the momentum / update buffers, no copies),
   1 multi-tensor launch   W <- f * decay * W - lr * scale * Phi  with the retraction factor f taken from sigma on the
                           device.

@@ -44,7 +44,9 @@ def msign(G: torch.Tensor, steps: int) -> torch.Tensor:
 def spectral_norm(w: torch.Tensor, steps: int = 50) -> torch.Tensor:
     """Top singular value of every matrix of ``w`` ([..., rows, cols], bf16 or fp32) by the vector sequence of the
     reference's power iteration (spectral_ball_utils.py:151-166), on the HIP path: one Gram matrix on the matrix
-    cores, then ``steps`` rounds of one launch each. Returns fp32 of shape ``w.shape[:-2]``; no host sync."""
+    cores (squared once / twice from 6 / 16 rounds on, so that one launch stands for two / four rounds; the last
+    application, whose quotient is the result, is the Gram matrix's). Returns fp32 of shape ``w.shape[:-2]``; no
+    host sync."""
     import ctypes
 
     from .. import _lib
