@@ -63,7 +63,7 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   // norm partials: one per 8192-element chunk (separate norm pass) or one per 64x64 tile of the padded matrix (fused pass)
   const size_t tiles64 = (size_t)(p.Mp / 64) * (p.Np / 64);
   p.off_partial = take((size_t)batch * std::max((size_t)p.cpm, tiles64) * sizeof(float));
-  p.off_scale = take((size_t)batch * sizeof(float));
+  p.off_scale = take((size_t)2 * batch * sizeof(float));   // deferred factor and the power of two applied to the copy
   p.total = off;
   return p;
 }
@@ -200,8 +200,9 @@ struct NsProblem {
   muon_ns_problem q;
   NsPlan pl;
   __bf16 *Xt[2], *A, *Bh, *Bl;   // Xt: the iterate as X^T, [b][Np][Mp] (long side first), ping-pong
-  float *partial, *scale;
+  float *partial, *scale, *pow2;
   bool tall;
+  bool defer;   // the operand of the first iteration is the input as it is; its epilogues apply 1/(|X| + eps)
   int sx;   // half-precision mode: the iterate is kept times 2^sx (its rms entry starts at about 2^-3)
 };
 
@@ -277,13 +278,26 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     P.Bl = split_any ? (__bf16*)(ws + P.pl.off_bl) : nullptr;
     P.partial = (float*)(ws + P.pl.off_partial);
     P.scale = (float*)(ws + P.pl.off_scale);
+    P.pow2 = P.scale + P.q.batch;
     P.tall = P.q.rows > P.q.cols;
+    // An input that is bfloat16 already (or is rounded to it before its norm) goes into the workspace EXACTLY and the
+    // factor is applied by the first iteration's epilogues, as after the fused momentum (all but a power of two, which
+    // the copy takes exactly and which keeps the products of the first iteration in range): rounding the normalised copy a
+    // second time is what a matrix with a few dominant singular values is sensitive to (Gaussian plus a 30x rank-one
+    // spike, error against an fp32 run: 5.2e-2 -> 5.0e-3 in bfloat16, 6.7e-3 -> 1.8e-3 with the half workspace).
+    P.defer = fused || (normalize && (P.q.in_dtype == MUON_DTYPE_BF16 || cast_first));
     P.sx = 0;
     if (f16) {
       const int l2 = (int)floor(0.5 * log2((double)P.pl.m * (double)P.pl.n)) - 3;
       P.sx = l2 > 0 ? l2 : 0;
     }
   }
+  // the half workspace starts with a bfloat16 iteration when the scale is deferred (see the iteration below); one
+  // kernel type per launch, so either every problem of the call defers or none does
+  bool defer_all = true;
+  for (const NsProblem& P : pr) defer_all = defer_all && P.defer;
+  if (f16 && !defer_all)
+    for (NsProblem& P : pr) P.defer = false;
   // launch order inside a grouped kernel: problems with the longest tiles first, so the tail of the
   // grid is made of short tiles
   std::vector<int> order(n_problems);
@@ -298,18 +312,19 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const NsProblem& P = pr[i];
     const NsPlan& pl = P.pl;
     const long xs = (long)pl.Mp * pl.Np;
-    const float* sc = normalize ? P.scale : nullptr;   // null: copy unscaled
+    const float* sc = !normalize ? nullptr : (P.defer ? P.pow2 : P.scale);   // null: copy unscaled
+    const int to_half = (f16 && !P.defer) ? 1 : 0;
     if (normalize) {
       e = launch_norm_scale(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                            P.q.cols, eps, eps_mode, P.partial, P.scale, stream);
+                            P.q.cols, eps, eps_mode, P.partial, P.scale, stream, P.defer ? P.pow2 : nullptr);
       if (e != hipSuccess) return (int)e;
     }
     if (!P.tall)
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, sc, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream, f16, P.sx);
+                        P.q.cols, sc, nullptr, 0, 0, pl.Mp, pl.Np, P.Xt[0], xs, pl.Mp, stream, to_half, to_half ? P.sx : 0);
     else
       e = launch_layout(P.q.in, P.q.in_dtype, cast_first, P.q.in_batch_stride, P.q.in_ld, P.q.batch, P.q.rows,
-                        P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream, f16, P.sx);
+                        P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream, to_half, to_half ? P.sx : 0);
     if (e != hipSuccess) return (int)e;
   }
   // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials
@@ -390,13 +405,13 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     // With the hi+lo pair the folded diagonal is exact; an iteration of a split call that keeps B in plain bf16 is not
     // folded (constant coefficients on small matrices: 8.4e-3 -> 1.1e-2 for 64x129 when it is).
     const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f && (!split_any || split);
-    // Half-precision workspace after the fused momentum: the unnormalised bfloat16 update cannot go into half as it is
-    // (its magnitude is the gradient's), so the first iteration runs on it in bfloat16 with the deferred scale, as in
-    // MUON_PREC_BF16, and its last product writes X' as scaled half.  The operand of that iteration is then the exact
+    // Half-precision workspace with a deferred scale (after the fused momentum, or a bfloat16 input): the unnormalised
+    // operand cannot go into half as it is (its magnitude is the gradient's), so the first iteration runs on it in
+    // bfloat16 with the deferred scale, as in MUON_PREC_BF16, and its last product writes X' as scaled half.  The operand of that iteration is then the exact
     // bfloat16 update, and A and B of ONE early iteration in bfloat16 cost nothing measurable (error against an fp32
     // run, CPU model, 512x2048 / 1024x1024 / 64x129: constant row 2.15 / 2.01 / 2.27e-3 against 2.16 / 2.03 / 2.22e-3
     // with all five iterations in half; a second bfloat16 iteration would cost 3.3 / 3.7 / 9.2e-3).
-    const bool lowp = f16 && fused && it == 0;
+    const bool lowp = f16 && defer_all && it == 0;
     const int SAi = lowp ? 0 : SA, SBi = lowp ? 0 : SB;
     const int ws16 = lowp ? 0 : (f16 ? 1 : 0);
     // A = X X^T, from X^T (K-major operand)
@@ -407,7 +422,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, SAi - 2 * (lowp ? 0 : P.sx)); g.beta = 0.f;
-      g.scale = (fused && it == 0) ? P.scale : nullptr;
+      g.scale = (P.defer && it == 0) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
@@ -441,7 +456,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.alpha = ldexpf(a, SBi); g.beta = 0.f;
       // the operand carries 2^sx (not in the bfloat16 iteration), the next iterate does, the caller's result does not
       g.out_shift = -SBi - (lowp ? 0 : P.sx) + ((last || !f16) ? 0 : P.sx);
-      g.scale = (fused && it == 0) ? P.scale : nullptr;
+      g.scale = (P.defer && it == 0) ? P.scale : nullptr;
       if (!last) {
         g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {

@@ -31,10 +31,11 @@ struct MomentumCoef {
 hipError_t launch_momentum(const PreItem* items, const int32_t* prefix, int n_items, int total_chunks,
                            MomentumCoef c, hipStream_t stream);
 
-// per-matrix Frobenius norms of in[batch][rows][cols] -> scale[b] = 1/(|X|+eps) or 1/max(|X|,eps)
+// per-matrix Frobenius norms of in[batch][rows][cols] -> scale[b] = 1/(|X|+eps) or 1/max(|X|,eps); with pow2 that
+// factor is split into pow2[b] (a power of two) times scale[b] (between 0.7 and 1.5)
 hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch,
                              int rows, int cols, float eps, int eps_mode, float* partial, float* scale,
-                             hipStream_t stream);
+                             hipStream_t stream, float* pow2 = nullptr);
 
 // D = bf16(scale*in) in the input's orientation and T = its transpose (either may be null), both zero-padded to
 // d_rows x d_cols / d_cols x d_rows (multiples of 64); scale may be null (= 1).  tile_sumsq (optional): the sum of

@@ -215,7 +215,7 @@ sumsq_partial_kernel(const void* __restrict__ in, long batch_stride, int rows, i
 
 __global__ void __launch_bounds__(EW_THREADS)
 norm_scale_kernel(const float* __restrict__ partial, int chunks_per_mat, float eps, int eps_mode,
-                  float* __restrict__ scale) {
+                  float* __restrict__ scale, float* __restrict__ pow2) {
   __shared__ float red[4];
   const int b = blockIdx.x;
   float s[1] = {0.f};
@@ -223,7 +223,16 @@ norm_scale_kernel(const float* __restrict__ partial, int chunks_per_mat, float e
   block_reduce<1>(s, red);
   if (threadIdx.x == 0) {
     const float n = sqrtf(s[0]);
-    scale[b] = eps_mode == EPS_ADD ? 1.f / (n + eps) : 1.f / fmaxf(n, eps);
+    const float sc = eps_mode == EPS_ADD ? 1.f / (n + eps) : 1.f / fmaxf(n, eps);
+    if (!pow2) {
+      scale[b] = sc;
+    } else {
+      // sc = pow2 * scale with pow2 a power of two (applied to the copy of the input, exactly) and scale in [0.7, 1.5]
+      const bool ok = sc > 0.f && sc < 3.0e38f;
+      const float p = ok ? exp2f(rintf(log2f(sc))) : sc;
+      pow2[b] = p;
+      scale[b] = ok ? sc / p : 1.f;
+    }
   }
 }
 
@@ -302,7 +311,7 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
 
 hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch,
                              int rows, int cols, float eps, int eps_mode, float* partial, float* scale,
-                             hipStream_t stream) {
+                             hipStream_t stream, float* pow2) {
   const long numel = (long)rows * cols;
   const int cpm = (int)((numel + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
   if (batch > 65535) return hipErrorInvalidValue;
@@ -315,7 +324,7 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
   else ARCHSCALE_SS(DT_F32, false);
 #undef ARCHSCALE_SS
   hipLaunchKernelGGL(norm_scale_kernel, dim3(batch), dim3(EW_THREADS), 0, stream, partial, cpm, eps, eps_mode,
-                     scale);
+                     scale, pow2);
   return hipGetLastError();
 }
 
@@ -458,7 +467,7 @@ hipError_t launch_norm_scale_from_partials(const float* partial, int partials_pe
                                            float* scale, hipStream_t stream) {
   if (batch < 1 || partials_per_mat < 1) return hipErrorInvalidValue;
   hipLaunchKernelGGL(norm_scale_kernel, dim3(batch), dim3(EW_THREADS), 0, stream, partial, partials_per_mat, eps, eps_mode,
-                     scale);
+                     scale, (float*)nullptr);
   return hipGetLastError();
 }
 

@@ -135,12 +135,14 @@ def newton_schulz(
     storage  "fp32":        bf16 input, every later op in fp32 (tolerance oracle)
              "bf16_eager":  every op on bf16 tensors, as the reference's CPU path
              "bf16_gemm":   one bf16 rounding per GEMM epilogue, the rounding
-                            points of newton_schulz_triton.py:374-378
+                            points of newton_schulz_triton.py:374-378; the normalised
+                            input itself is NOT rounded again (the HIP path keeps the
+                            bf16 input exactly and applies the factor in fp32)
              "bf16_gemm_bsplit": as bf16_gemm but B kept as a bf16 hi+lo pair
              "f16_gemm":    a model of the HIP path's half-precision workspace (no counterpart in the reference): one
                             IEEE-half rounding per GEMM epilogue with X, A, B kept times 2^sx, 2^8, 2^6
                             (sx = floor(log2 sqrt(m n)) - 3), a*I inside B after the first iteration where |a| <= 4.2,
-                            bf16 result
+                            bf16 result; the first iteration runs on the exact input with A and B in bf16
     Returns bf16 for the bf16 / f16 modes and fp32 for "fp32", shaped like G.
     """
     if G.ndim < 2:
@@ -167,7 +169,6 @@ def newton_schulz(
                 B = b * A + c * (A @ A)
                 X = a * X + B @ X
         elif storage in ("bf16_gemm", "bf16_gemm_bsplit"):
-            X = _bf16_round(X)
             for a, b, c in coeffs:
                 A = _bf16_round(X @ X.mT)
                 B = c * (A @ A) + b * A
@@ -185,16 +186,16 @@ def newton_schulz(
             def half(t: Tensor, shift: int) -> Tensor:
                 return (t * 2.0 ** shift).to(torch.float16).to(torch.float32) * 2.0 ** -shift
 
-            X = half(X, sx)
             eye = torch.eye(m, dtype=torch.float32)
             for it, (a, b, c) in enumerate(coeffs):
-                A = half(X @ X.mT, 8)
+                first = it == 0
+                A = _bf16_round(X @ X.mT) if first else half(X @ X.mT, 8)
                 B = c * (A @ A) + b * A
                 last = it == len(coeffs) - 1
                 if it > 0 and abs(a) <= 4.2:
                     Y = half(B + a * eye, 6) @ X
                 else:
-                    Y = a * X + half(B, 6) @ X
+                    Y = a * X + (_bf16_round(B) if first else half(B, 6)) @ X
                 X = _bf16_round(Y) if last else half(Y, sx)
             X = X.to(torch.bfloat16)
         else:
