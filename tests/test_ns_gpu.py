@@ -282,6 +282,36 @@ def test_dominant_singular_value(ns, gpu_device):
     assert _rel(got, rounded) <= 3e-2
 
 
+@pytest.mark.parametrize("prec", ["bf16", "f16"])
+def test_power_of_two_scaling_is_exact(ns, gpu_device, prec):
+    """A bf16 input goes into the workspace times a power of two and the rest of 1/|X| is applied in fp32, so a matrix
+    times 2^k (exact in bf16) must give the same bits as the matrix itself when eps is zero, for tiny and huge k."""
+    G = _randn((200, 330), 77).to(torch.bfloat16)
+    coeffs = O.coefficient_schedule("quintic", 5)
+    base = ns.newton_schulz(G.to(gpu_device), coeffs, 0.0, prec=prec)
+    assert _rel(base, O.newton_schulz(G, coeffs, 0.0, storage="fp32")) <= (4e-3 if prec == "f16" else NS_TOL)
+    for k in (-40, -13, 9, 30):
+        got = ns.newton_schulz((G.float() * 2.0 ** k).to(torch.bfloat16).to(gpu_device), coeffs, 0.0, prec=prec)
+        assert torch.equal(got, base), k
+
+
+def test_grouped_call_with_mixed_input_kinds(ns, gpu_device):
+    """One grouped call over a bf16 tensor (kept exactly, factor deferred) and an fp32 tensor that is normalised before
+    it is rounded (not deferrable): in bf16 storage each problem takes its own route, with the half workspace the whole
+    call takes the common one; every result stays within its bar of the fp32 run."""
+    coeffs = O.coefficient_schedule("quintic", 5)
+    a = _randn((2, 128, 320), 5).to(torch.bfloat16)
+    b = _randn((192, 96), 6)
+    want_a = O.newton_schulz(a, coeffs, 1e-7, storage="fp32")
+    want_b = O.newton_schulz(b, coeffs, 1e-7, storage="fp32")   # the oracle rounds first; the difference is one rounding
+    for prec, bar in (("bf16", NS_TOL), ("f16", 4e-3)):
+        got_a, got_b = ns.newton_schulz_grouped([a.to(gpu_device), b.to(gpu_device)], coeffs, 1e-7, prec=prec,
+                                                cast_input_first=False)
+        torch.cuda.synchronize()
+        print(prec, _rel(got_a, want_a), _rel(got_b, want_b), flush=True)
+        assert _rel(got_a, want_a) <= bar and _rel(got_b, want_b) <= NS_TOL
+
+
 def test_random_shapes_strides_and_modes(ns, gpu_device):
     """Seeded sweep over shapes that are no multiple of anything, strided inputs, both input dtypes, all coefficient
     tables, split tails, the no-fold flag and grouped calls of mixed size: every result within the bar of the fp32 run,
