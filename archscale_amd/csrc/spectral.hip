@@ -192,7 +192,9 @@ sn_xscale_kernel(const SnParams sp) {
   for (int i = threadIdx.x; i < c.xtiles; i += 64) t += part[i];
   t = wave_sum(t);
   // a power of two: X and G are scaled exactly
-  if (threadIdx.x == 0) c.xscale[blk] = t > 0.f ? exp2f(rintf(0.5f * log2f((float)c.d / t))) : 0.f;
+  // (exponent clamped: xscale^2 multiplies an fp32 accumulator)
+  if (threadIdx.x == 0)
+    c.xscale[blk] = t > 0.f ? exp2f(fminf(fmaxf(rintf(0.5f * log2f((float)c.d / t)), -60.f), 60.f)) : 0.f;
 }
 
 int spectral_power_levels(int steps) {
