@@ -60,7 +60,7 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   p.off_a = take(ab);
   p.off_bh = take(ab);
   p.off_bl = prec_mode == MUON_PREC_BF16_BSPLIT ? take(ab) : 0;
-  // norm partials: one per 8192-element chunk (separate norm pass) or one per 64x64 tile of the padded matrix (fused pass)
+  // norm partials: one per 8192-element chunk (separate norm pass) or one per tile of the fused momentum pass (at most one per 64x64 elements)
   const size_t tiles64 = (size_t)(p.Mp / 64) * (p.Np / 64);
   p.off_partial = take((size_t)batch * std::max((size_t)p.cpm, tiles64) * sizeof(float));
   p.off_scale = take((size_t)2 * batch * sizeof(float));   // deferred factor and the power of two applied to the copy
@@ -334,7 +334,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const muon_mns_problem& f = fused[i];
     const long xs = (long)pl.Mp * pl.Np;
     const int d_rows = P.tall ? pl.Np : pl.Mp, d_cols = P.tall ? pl.Mp : pl.Np;   // padded extents of the matrix itself
-    const int tiles = (d_rows / 64) * (d_cols / 64);
+    const int tiles = (d_rows / MOMLAY_TILE) * (d_cols / MOMLAY_TILE);
     for (int b0 = 0; b0 < P.q.batch; b0 += MOMLAY_MAX) {
       MomLayoutParams mp = {};
       mp.n_mats = std::min(MOMLAY_MAX, P.q.batch - b0);

@@ -47,15 +47,16 @@ hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_b
 
 // momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
 constexpr int MOMLAY_MAX = 32;
+constexpr int MOMLAY_TILE = 128;   // rows and columns of the tile of one block; one partial sum per tile
 struct MomLayoutParams {
   int n_mats, rows, cols;        // matrices of this launch, all rows x cols, contiguous
   int g_dtype, m_dtype, w_dtype;
   int transpose;                 // dst holds the transpose of the matrix (d_cols x d_rows) instead of the matrix
-  int d_rows, d_cols;            // extents of the matrix padded to multiples of 64 (the grid)
+  int d_rows, d_cols;            // extents of the matrix padded to multiples of MOMLAY_TILE (the grid)
   int ldd;                       // leading dimension of dst
   long d_bstride;                // elements between consecutive matrices in dst
   uint16_t* dst;                 // bf16
-  float* partial;                // [n_mats][(d_rows/64) * (d_cols/64)] sums of squares
+  float* partial;                // [n_mats][(d_rows/MOMLAY_TILE) * (d_cols/MOMLAY_TILE)] sums of squares
   MomentumCoef c;
   const void* g[MOMLAY_MAX];
   void* m[MOMLAY_MAX];

@@ -352,80 +352,100 @@ hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_b
 //     normalisation 1/(|U| + eps) is applied by the first iteration's GEMM epilogues.  One launch covers up to
 //     MOMLAY_MAX matrices of one shape (their tensors are separate allocations: pointers by value).
 // ---------------------------------------------------------------------------
+// tile of one block: MOMLAY_TILE x MOMLAY_TILE elements, so that a row of it is 256 contiguous bytes in the source and
+// in either destination image
+constexpr int MOMLAY_TPR = MOMLAY_TILE / 8;          // threads per tile row (8 elements each)
+constexpr int MOMLAY_RPP = 256 / MOMLAY_TPR;         // tile rows per pass of the block
+constexpr int MOMLAY_PASSES = MOMLAY_TILE / MOMLAY_RPP;
+constexpr int MOMLAY_BATCH = 4;                      // passes whose loads are issued before any of their stores
+
 template <int GD, int MD>
-__device__ __forceinline__ void momlay_tile(const MomLayoutParams& p, int mat, int r0, int c0, uint16_t (&tile)[64][66],
-                                            float& sumsq) {
+__device__ __forceinline__ void momlay_tile(const MomLayoutParams& p, int mat, int r0, int c0,
+                                            uint16_t (&tile)[MOMLAY_TILE][MOMLAY_TILE + 2], float& sumsq) {
   const char* g = (const char*)p.g[mat];
   char* m = (char*)p.m[mat];
   const void* w = p.w[mat];
-  const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
+  const int tr = threadIdx.x / MOMLAY_TPR, tc = (threadIdx.x % MOMLAY_TPR) * 8;
+  const int c = c0 + tc;
   const bool vec = aligned16(g) && aligned16(m) && (p.cols % 8 == 0) && (p.c.l2 == 0.f || aligned16(w));
+  const bool cols_in = vec && c + 7 < p.cols;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int r = r0 + tr + h * 32, c = c0 + tc;
-    float uv[8];
-    if (r < p.rows && c + 7 < p.cols && vec) {
-      const long i = (long)r * p.cols + c;
-      float gv[8], mv[8];
-      Elem<GD>::load8(g, i, gv);
-      Elem<MD>::load8(m, i, mv);
-      if (p.c.l2 != 0.f) {
-        float wv[8];
-        if (p.w_dtype == DT_BF16) Elem<DT_BF16>::load8(w, i, wv); else Elem<DT_F32>::load8(w, i, wv);
+  for (int hb = 0; hb < MOMLAY_PASSES; hb += MOMLAY_BATCH) {
+    // all loads of the batch first: the stores below may alias them as far as the compiler knows
+    float gv[MOMLAY_BATCH][8], mv[MOMLAY_BATCH][8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) gv[k] = Elem<GD>::round(gv[k] + p.c.l2 * wv[k]);
-        Elem<GD>::store8(const_cast<char*>(g), i, gv);
+    for (int j = 0; j < MOMLAY_BATCH; ++j) {
+      const int r = r0 + tr + (hb + j) * MOMLAY_RPP;
+      if (r < p.rows && cols_in) {
+        const long i = (long)r * p.cols + c;
+        Elem<GD>::load8(g, i, gv[j]);
+        Elem<MD>::load8(m, i, mv[j]);
       }
+    }
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const float gm = Elem<MD>::round(gv[k]);
-        const float mn = Elem<MD>::round(fmaf(p.c.mm, mv[k], p.c.mg * gm));
-        mv[k] = mn;
-        uv[k] = fmaf(p.c.um, mn, p.c.ug * gm);
-      }
-      Elem<MD>::store8(m, i, mv);
-    } else {
+    for (int j = 0; j < MOMLAY_BATCH; ++j) {
+      const int r = r0 + tr + (hb + j) * MOMLAY_RPP;
+      float uv[8];
+      if (r < p.rows && cols_in) {
+        const long i = (long)r * p.cols + c;
+        if (p.c.l2 != 0.f) {
+          float wv[8];
+          if (p.w_dtype == DT_BF16) Elem<DT_BF16>::load8(w, i, wv); else Elem<DT_F32>::load8(w, i, wv);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        uv[k] = 0.f;
-        if (r < p.rows && c + k < p.cols) {
-          const long i = (long)r * p.cols + c + k;
-          float gv = Elem<GD>::load1(g, i);
-          if (p.c.l2 != 0.f) {
-            const float wv = p.w_dtype == DT_BF16 ? Elem<DT_BF16>::load1(w, i) : Elem<DT_F32>::load1(w, i);
-            gv = Elem<GD>::round(gv + p.c.l2 * wv);
-            Elem<GD>::store1(const_cast<char*>(g), i, gv);
-          }
-          const float gm = Elem<MD>::round(gv);
-          const float mn = Elem<MD>::round(fmaf(p.c.mm, Elem<MD>::load1(m, i), p.c.mg * gm));
-          Elem<MD>::store1(m, i, mn);
+          for (int k = 0; k < 8; ++k) gv[j][k] = Elem<GD>::round(gv[j][k] + p.c.l2 * wv[k]);
+          Elem<GD>::store8(const_cast<char*>(g), i, gv[j]);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float gm = Elem<MD>::round(gv[j][k]);
+          const float mn = Elem<MD>::round(fmaf(p.c.mm, mv[j][k], p.c.mg * gm));
+          mv[j][k] = mn;
           uv[k] = fmaf(p.c.um, mn, p.c.ug * gm);
         }
-      }
-    }
-    uint16_t o[8];
+        Elem<MD>::store8(m, i, mv[j]);
+      } else {
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      o[k] = f2bf(uv[k]);
-      const float x = bf2f(o[k]);
-      sumsq += x * x;
-      tile[tr + h * 32][tc + k] = o[k];
-    }
-    if (!p.transpose) {
-      uint4 pk;
-      pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
-      pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
-      *(uint4*)(p.dst + (size_t)mat * p.d_bstride + (size_t)r * p.ldd + c) = pk;
+        for (int k = 0; k < 8; ++k) {
+          uv[k] = 0.f;
+          if (r < p.rows && c + k < p.cols) {
+            const long i = (long)r * p.cols + c + k;
+            float gs = Elem<GD>::load1(g, i);
+            if (p.c.l2 != 0.f) {
+              const float wv = p.w_dtype == DT_BF16 ? Elem<DT_BF16>::load1(w, i) : Elem<DT_F32>::load1(w, i);
+              gs = Elem<GD>::round(gs + p.c.l2 * wv);
+              Elem<GD>::store1(const_cast<char*>(g), i, gs);
+            }
+            const float gm = Elem<MD>::round(gs);
+            const float mn = Elem<MD>::round(fmaf(p.c.mm, Elem<MD>::load1(m, i), p.c.mg * gm));
+            Elem<MD>::store1(m, i, mn);
+            uv[k] = fmaf(p.c.um, mn, p.c.ug * gm);
+          }
+        }
+      }
+      uint16_t o[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        o[k] = f2bf(uv[k]);
+        const float x = bf2f(o[k]);
+        sumsq += x * x;
+        tile[tr + (hb + j) * MOMLAY_RPP][tc + k] = o[k];
+      }
+      if (!p.transpose) {
+        uint4 pk;
+        pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
+        pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
+        *(uint4*)(p.dst + (size_t)mat * p.d_bstride + (size_t)r * p.ldd + c) = pk;
+      }
     }
   }
 }
 
 __global__ void __launch_bounds__(256)
 momentum_layout_kernel(const MomLayoutParams p) {
-  __shared__ uint16_t tile[64][66];
+  __shared__ uint16_t tile[MOMLAY_TILE][MOMLAY_TILE + 2];
   __shared__ float red[4];
   const int mat = blockIdx.z;
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;   // tile of the padded source orientation (d_rows x d_cols)
+  const int r0 = blockIdx.y * MOMLAY_TILE, c0 = blockIdx.x * MOMLAY_TILE;   // tile of the padded source orientation
   float s[1] = {0.f};
   const int key = (p.g_dtype << 1) | p.m_dtype;
   switch (key) {
@@ -436,14 +456,14 @@ momentum_layout_kernel(const MomLayoutParams p) {
   }
   __syncthreads();
   if (p.transpose) {
-    const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
+    const int tr = threadIdx.x / MOMLAY_TPR, tc = (threadIdx.x % MOMLAY_TPR) * 8;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int c = c0 + tr + h * 32;   // row of the transposed image
-      const int r = r0 + tc;            // 8 consecutive columns of it
+    for (int h = 0; h < MOMLAY_PASSES; ++h) {
+      const int c = c0 + tr + h * MOMLAY_RPP;   // row of the transposed image
+      const int r = r0 + tc;                    // 8 consecutive columns of it
       uint16_t o[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) o[k] = tile[tc + k][tr + h * 32];
+      for (int k = 0; k < 8; ++k) o[k] = tile[tc + k][tr + h * MOMLAY_RPP];
       uint4 pk;
       pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
       pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
@@ -455,10 +475,11 @@ momentum_layout_kernel(const MomLayoutParams p) {
 }
 
 hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream) {
-  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.d_rows % 64 || p.d_cols % 64 || p.d_rows / 64 > 65535 ||
-      p.rows > p.d_rows || p.cols > p.d_cols || p.rows < 1 || p.cols < 1)
+  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.d_rows % MOMLAY_TILE || p.d_cols % MOMLAY_TILE ||
+      p.d_rows / MOMLAY_TILE > 65535 || p.rows > p.d_rows || p.cols > p.d_cols || p.rows < 1 || p.cols < 1)
     return hipErrorInvalidValue;
-  hipLaunchKernelGGL(momentum_layout_kernel, dim3(p.d_cols / 64, p.d_rows / 64, p.n_mats), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL(momentum_layout_kernel, dim3(p.d_cols / MOMLAY_TILE, p.d_rows / MOMLAY_TILE, p.n_mats), dim3(256), 0,
+                     stream, p);
   return hipGetLastError();
 }
 
