@@ -25,6 +25,7 @@ NS_CAST_INPUT_FIRST = 1
 NS_NO_NORMALIZE = 2
 NS_NO_DIAG_FOLD = 4
 CHUNK_ELEMS = 8192
+PROF_KEY_MOMENTUM_LAYOUT = 90000
 ABI_VERSION = 2
 
 #: numpy layouts of muon_pre_item / muon_post_item (natural C alignment)
@@ -247,8 +248,9 @@ def profile_begin() -> None:
 
 def profile_collect(capacity: int = 4096):
     """Per-launch records of the Newton-Schulz GEMMs since profile_begin():
-    list of dicts {ms, tile, mode, split, final, folded, flops_algorithmic, flops_issued}; ``folded`` marks the
-    X' = (B + aI) X launches that read no addend."""
+    list of dicts {kind="gemm", ms, tile, mode, split, final, folded, flops_algorithmic, flops_issued} (``folded`` marks
+    the X' = (B + aI) X launches that read no addend) and {kind="momentum_layout", ms, bytes} for the fused momentum
+    launches (``bytes`` = algorithmic HBM bytes of the launch)."""
     ms = (ctypes.c_float * capacity)()
     key = (ctypes.c_int32 * capacity)()
     fa = (ctypes.c_double * capacity)()
@@ -259,6 +261,9 @@ def profile_collect(capacity: int = 4096):
     out = []
     for i in range(min(n, capacity)):
         k = key[i]
-        out.append(dict(ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool((k % 10) & 2), final=bool((k % 10) & 1), folded=bool((k % 10) & 4),
-                        flops_algorithmic=fa[i], flops_issued=fi[i]))
+        if k == PROF_KEY_MOMENTUM_LAYOUT:   # the fused momentum launch: the work fields carry bytes
+            out.append(dict(kind="momentum_layout", ms=ms[i], bytes=fa[i]))
+            continue
+        out.append(dict(kind="gemm", ms=ms[i], tile=k // 100, mode=(k // 10) % 10, split=bool((k % 10) & 2),
+                        final=bool((k % 10) & 1), folded=bool((k % 10) & 4), flops_algorithmic=fa[i], flops_issued=fi[i]))
     return out

@@ -77,47 +77,56 @@ size_t plan_bytes_bound(int batch, int rows, int cols, int prec_mode) {
   return std::max(make_plan(batch, rows, cols, prec_mode, 256).total, make_plan(batch, rows, cols, prec_mode, 128).total);
 }
 
+constexpr int MAX_DEVICES = 64;
+
+// compute units of the CURRENT device (cached per device; a racing first call only repeats the query)
 int compute_units() {
-  static const int n = [] {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      return v;
-    return 256;
-  }();
-  return n;
+  static std::atomic<int> cached[MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  const bool slot = dev >= 0 && dev < MAX_DEVICES;
+  int v = slot ? cached[dev].load(std::memory_order_relaxed) : 0;
+  if (v > 0) return v;
+  if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 256;
+  if (slot) cached[dev].store(v, std::memory_order_relaxed);
+  return v;
 }
 
-// Optional per-launch timing of the Newton-Schulz GEMMs (muon_profile_begin / muon_profile_collect):
-// one pair of HIP events around every GEMM launch, on the stream the kernel runs on.
+// Optional per-launch timing (muon_profile_begin / muon_profile_collect): one pair of HIP events around every
+// Newton-Schulz GEMM launch and every fused momentum launch, on the stream the kernel runs on.  The events come from a
+// pool that muon_profile_begin creates, so a timed call creates nothing; launches beyond the pool run untimed.
+// Profiling is a single-threaded debugging mode: every timed launch takes one process-wide lock.
 struct ProfRec {
-  hipEvent_t start, stop;
-  int key;  // tile*100 + mode*10 + 4*(BX without addend) + split*2 + final
-  double flops_algorithmic, flops_issued;
+  int key;  // tile*100 + mode*10 + 4*(BX without addend) + split*2 + final; PROF_KEY_MOMENTUM_LAYOUT for the fused momentum
+  double work_algorithmic, work_issued;   // FLOPs of a GEMM launch; bytes of a momentum launch
 };
+constexpr int PROF_POOL = 1024;
+constexpr int PROF_KEY_MOMENTUM_LAYOUT = 90000;
 std::mutex g_prof_mutex;
-std::vector<ProfRec> g_prof;
+std::vector<hipEvent_t> g_prof_start, g_prof_stop;   // the pool
+std::vector<ProfRec> g_prof;                         // g_prof[i] used events i
 std::atomic<bool> g_prof_on{false};
+
+// runs `launch` between two pooled events when profiling is on
+template <class F>
+hipError_t timed_launch(int key, double work_algorithmic, double work_issued, hipStream_t stream, F&& launch) {
+  if (!g_prof_on.load(std::memory_order_acquire)) return launch();
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  const size_t i = g_prof.size();
+  if (!g_prof_on || i >= g_prof_start.size()) return launch();
+  hipError_t e = hipEventRecord(g_prof_start[i], stream);
+  if (e != hipSuccess) return e;
+  e = launch();
+  const hipError_t e2 = hipEventRecord(g_prof_stop[i], stream);
+  g_prof.push_back(ProfRec{key, work_algorithmic, work_issued});
+  return e != hipSuccess ? e : e2;
+}
 
 hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const GroupedGemmParams& g, hipStream_t stream,
                       double flops_algorithmic, double flops_issued, int f16 = 0) {
-  if (!g_prof_on) return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16);
-  std::lock_guard<std::mutex> lock(g_prof_mutex);
-  ProfRec r;
-  r.key = tile * 100 + mode * 10 + ((mode == MODE_BX && !g.g[0].E) ? 4 : 0) + (split ? 2 : 0) + (final_ ? 1 : 0);
-  r.flops_algorithmic = flops_algorithmic;
-  r.flops_issued = flops_issued;
-  hipError_t e;
-  if ((e = hipEventCreate(&r.start)) != hipSuccess) return e;
-  if ((e = hipEventCreate(&r.stop)) != hipSuccess) { (void)hipEventDestroy(r.start); return e; }
-  if ((e = hipEventRecord(r.start, stream)) != hipSuccess) {
-    (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop);
-    return e;
-  }
-  e = launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16);
-  hipError_t e2 = hipEventRecord(r.stop, stream);
-  g_prof.push_back(r);
-  return e != hipSuccess ? e : e2;
+  const int key = tile * 100 + mode * 10 + ((mode == MODE_BX && !g.g[0].E) ? 4 : 0) + (split ? 2 : 0) + (final_ ? 1 : 0);
+  return timed_launch(key, flops_algorithmic, flops_issued, stream,
+                      [&] { return launch_ns_gemm_grouped(tile, mode, split, final_, g, stream, f16); });
 }
 
 // One product over all problems of a 256-tile launch.  When the last round of the grid would hold only a few tiles, the
@@ -350,7 +359,11 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
         mp.m[k] = f.m_ptrs[b0 + k];
         mp.w[k] = f.w_ptrs ? f.w_ptrs[b0 + k] : nullptr;
       }
-      if ((e = launch_momentum_layout(mp, stream)) != hipSuccess) return (int)e;
+      // algorithmic bytes: G read, M read and written, the operand image written (2 bytes each)
+      const double esz = (double)mp.n_mats * P.q.rows * P.q.cols;
+      const double bytes = esz * ((f.g_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2 * (f.m_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2);
+      e = timed_launch(PROF_KEY_MOMENTUM_LAYOUT, bytes, bytes, stream, [&] { return launch_momentum_layout(mp, stream); });
+      if (e != hipSuccess) return (int)e;
     }
     e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);
     if (e != hipSuccess) return (int)e;
@@ -765,29 +778,35 @@ int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void
 
 int muon_profile_begin(void) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
-  for (auto& r : g_prof) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
   g_prof.clear();
-  g_prof_on = true;
+  while ((int)g_prof_start.size() < PROF_POOL) {
+    hipEvent_t a, b;
+    hipError_t e = hipEventCreate(&a);
+    if (e != hipSuccess) return (int)e;
+    if ((e = hipEventCreate(&b)) != hipSuccess) { (void)hipEventDestroy(a); return (int)e; }
+    g_prof_start.push_back(a);
+    g_prof_stop.push_back(b);
+  }
+  g_prof.reserve(PROF_POOL);
+  g_prof_on.store(true, std::memory_order_release);
   return 0;
 }
 
 int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algorithmic_host,
                          double* flops_issued_host, int capacity) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
-  g_prof_on = false;
+  g_prof_on.store(false, std::memory_order_release);
   int n = 0;
-  for (auto& r : g_prof) {
+  for (size_t i = 0; i < g_prof.size(); ++i) {
     float ms = 0.f;
-    hipError_t e = hipEventSynchronize(r.stop);
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.start, r.stop);
-    (void)hipEventDestroy(r.start);
-    (void)hipEventDestroy(r.stop);
+    hipError_t e = hipEventSynchronize(g_prof_stop[i]);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, g_prof_start[i], g_prof_stop[i]);
     if (e != hipSuccess) { g_prof.clear(); return -(int)e - 1000; }
     if (n < capacity) {
       if (ms_host) ms_host[n] = ms;
-      if (key_host) key_host[n] = r.key;
-      if (flops_algorithmic_host) flops_algorithmic_host[n] = r.flops_algorithmic;
-      if (flops_issued_host) flops_issued_host[n] = r.flops_issued;
+      if (key_host) key_host[n] = g_prof[i].key;
+      if (flops_algorithmic_host) flops_algorithmic_host[n] = g_prof[i].work_algorithmic;
+      if (flops_issued_host) flops_issued_host[n] = g_prof[i].work_issued;
     }
     ++n;
   }

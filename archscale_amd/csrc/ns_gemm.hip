@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "ns_gemm.h"
@@ -244,25 +245,42 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   static_assert(G1 == 4 || G1 == 8 || G1 == 16, "the first wait below is written for these counts");
   bf16x8 af[2][FM], bq[2][FN];
   // The transpose reads are inline assembly: the compiler makes the builtin wait for every outstanding global->LDS
-  // copy (vmcnt(0)) before each read.  Their results are therefore not tracked by the compiler; an explicit
-  // s_waitcnt lgkmcnt(0), fenced, precedes the first MFMA of every k-step.
-  auto tr8 = [&](const char* base, int pitch, int kk) {
-    unsigned long long lo, hi4;
+  // copy (vmcnt(0)) before each read.  The compiler therefore does not know that their results arrive late.  The raw
+  // results stay in variables of their own (afr / bqr, one 64-bit pair per read) that nothing touches until the explicit
+  // s_waitcnt lgkmcnt(0) before the first MFMA of the k-step; that wait is followed by empty asm statements that take
+  // every raw result as a read-write operand, so each use (the packing into an MFMA operand included) depends on a
+  // statement that comes after the wait.
+  typedef unsigned long long u64;
+  u64 afr[2][KMAJ ? FM : 1][2], bqr[2][KMAJ ? FN : 1][2];
+  auto tr8 = [&](const char* base, int pitch, int kk, u64 (&raw)[2]) {
     const uint32_t a0 = (uint32_t)(uintptr_t)base + (uint32_t)(16 * kk * pitch);
     const uint32_t a1 = a0 + (uint32_t)(4 * pitch);
-    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a0));
-    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi4) : "v"(a1));
-    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
-    const u64x2 v = {lo, hi4};
-    return __builtin_bit_cast(bf16x8, v);
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(raw[0]) : "v"(a0));
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(raw[1]) : "v"(a1));
   };
   auto fread = [&](int buf, const char* sP, const char* sQ, int kk, int r) {
     if constexpr (!KMAJ) {
       if (r < FM) af[buf][r] = *(const bf16x8*)(sP + rdP[kk] + r * 32 * ROW_BYTES);
       else bq[buf][r - FM] = *(const bf16x8*)(sQ + rdQ[kk] + (r - FM) * 32 * ROW_BYTES);
     } else {
-      if (r < FM) af[buf][r] = tr8(sP + trP[r], BM * 2, kk);
-      else bq[buf][r - FM] = tr8(sQ + trQ[r - FM], BN * 2, kk);
+      if (r < FM) tr8(sP + trP[r], BM * 2, kk, afr[buf][r]);
+      else tr8(sQ + trQ[r - FM], BN * 2, kk, bqr[buf][r - FM]);
+    }
+  };
+  // K-major operands: wait for the transpose reads of fragment buffer `buf`, then pack them
+  auto land = [&](int buf) {
+    if constexpr (KMAJ) {
+      typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < FM; ++i) asm volatile("" : "+v"(afr[buf][i][0]), "+v"(afr[buf][i][1]));
+#pragma unroll
+      for (int j = 0; j < FN; ++j) asm volatile("" : "+v"(bqr[buf][j][0]), "+v"(bqr[buf][j][1]));
+#pragma unroll
+      for (int i = 0; i < FM; ++i) { const u64x2 v = {afr[buf][i][0], afr[buf][i][1]}; af[buf][i] = __builtin_bit_cast(bf16x8, v); }
+#pragma unroll
+      for (int j = 0; j < FN; ++j) { const u64x2 v = {bqr[buf][j][0], bqr[buf][j][1]}; bq[buf][j] = __builtin_bit_cast(bf16x8, v); }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // one k-step: MFMAs on fragment buffer CBUF (when COMPUTE), reads of k-step RKK of the stage at (rP, rQ)
@@ -272,10 +290,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     constexpr bool COMPUTE = decltype(compute)::value, READ = decltype(read)::value;
     constexpr int cbuf = decltype(cbuf_)::value, rbuf = decltype(rbuf_)::value, rkk = decltype(rkk_)::value;
     constexpr int g0 = decltype(g0_)::value, g1 = decltype(g1_)::value;
-    if constexpr (KMAJ && COMPUTE) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    if constexpr (COMPUTE) land(cbuf);
 #pragma unroll
     for (int q = 0; q < NMF; ++q) {
       if (COMPUTE)
@@ -707,16 +722,17 @@ static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
   auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>;
-  // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device
-  // (idempotent; a benign race only repeats the call)
-  static bool attr_set[64] = {};
+  // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device and instantiation
+  // (the call is idempotent, so two threads that race on the first launch only repeat it)
+  static std::atomic<bool> attr_set[64];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev < 0 || dev >= 64 || !attr_set[dev]) {
+  const bool slot = dev >= 0 && dev < 64;
+  if (!slot || !attr_set[dev].load(std::memory_order_acquire)) {
     e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) attr_set[dev] = true;
+    if (slot) attr_set[dev].store(true, std::memory_order_release);
   }
   const long tiles = gp.tile_start[gp.n_groups];
   if (tiles <= 0) return hipSuccess;

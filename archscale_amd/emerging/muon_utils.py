@@ -39,16 +39,16 @@ def newton_schulz(x: torch.Tensor, steps: int, coefficient_type: str = "polar_ex
                   custom_coefficient_sets=None, eps: float = 1e-7, transpose=None, tp_group=None,
                   use_syrk: bool = False) -> torch.Tensor:
     """fp32 in, fp32 out; the set is cycled ``i % len(set)`` and ``steps`` must be a multiple of its length.
-    ``use_syrk`` is accepted and ignored (the HIP path always computes only the upper triangle);
-    ``transpose`` may only confirm the automatic choice; tensor-parallel groups are not supported here."""
+    ``use_syrk`` is accepted and ignored (the HIP path always computes only the upper triangle).  ``transpose`` is
+    accepted and has no effect: the iteration acts on the singular values only, so iterating on the matrix or on its
+    transpose gives the same result, and the library always iterates with the short side first.  Tensor-parallel
+    groups are not supported here."""
     if x.ndim < 2:
         raise ValueError("Input tensor x must have at least 2 dimensions since Muon is not for 1d parameters.")
     if x.dtype != torch.float32:
         raise ValueError(f"Input tensor x must be in float32, got {x.dtype}")
     if tp_group is not None:
         raise NotImplementedError("this build runs Newton-Schulz on one GPU; tp_group must be None")
-    if transpose is not None and bool(transpose) != (x.size(-2) > x.size(-1)):
-        raise NotImplementedError("only the automatic transpose (rows > cols) is supported")
     if coefficient_type in _COEFFICIENT_SETS:
         sets = _COEFFICIENT_SETS[coefficient_type]
     elif coefficient_type == "custom":

@@ -85,10 +85,115 @@ def cpu_baseline(coeffs_name, seed, budget_s=15.0):
     }
 
 
+def _gemm_summary(recs):
+    """(ms, issued FLOPs, algorithmic FLOPs) summed over the GEMM launches of one instrumented call."""
+    gem = [r for r in recs if r["kind"] == "gemm"]
+    return (sum(r["ms"] for r in gem), sum(r["flops_issued"] for r in gem), sum(r["flops_algorithmic"] for r in gem))
+
+
+def _time_calls(fn, reps, warm=2):
+    """Average milliseconds of `fn` over `reps` back-to-back calls on the current stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def _instrumented(fn):
+    from archscale_amd import _lib
+    _lib.profile_begin()
+    fn()
+    torch.cuda.synchronize()
+    return _lib.profile_collect()
+
+
+def other_configs(dev, which):
+    """The remaining benchmark configurations (1, 3, 4, 5) on the same code paths as the GPU tests: seeded synthetic
+    inputs generated on the device, each timed by HIP events over several back-to-back calls, plus one instrumented call
+    for the share of the bf16 matrix-core peak that the GEMM launches reach (issued FLOPs over their summed durations)."""
+    from archscale_amd import _lib
+    from archscale_amd.optim.muon import Muon
+    import archscale_amd.optim.newton_schulz_hip as H
+    out = {}
+
+    def gen(shape, seed, scale):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return (torch.randn(*shape, generator=g, device=dev) * scale).to(torch.bfloat16)
+
+    def pack(ms, shapes_counts, recs, **extra):
+        dense = sum(c * dense_flops(s) for s, c in shapes_counts)
+        gms, fi, fa = _gemm_summary(recs)
+        d = {"ms": round(ms, 4), "dense_tflops": round(dense / ms / 1e9, 1),
+             "gemm_ms": round(gms, 4),
+             "gemm_pct_mfma_peak_issued": round(fi / gms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2) if gms else None,
+             "gemm_pct_mfma_peak_algorithmic": round(fa / gms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2) if gms else None}
+        d.update(extra)
+        return d
+
+    def muonh_step_config(shapes, seed, reps):
+        params = [torch.nn.Parameter(gen(s, seed + 2 * i, 0.02)) for i, s in enumerate(shapes)]
+        for i, p in enumerate(params):
+            p.grad = gen(tuple(p.shape), seed + 2 * i + 1, 1e-3)
+        opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, use_muonh=True,
+                   muonh_per_matrix=True)
+        ms = _time_calls(opt.step, reps)
+        recs = _instrumented(opt.step)
+        return ms, recs, sum(p.numel() for p in params)
+
+    if 1 in which:   # one 512x2048 gradient, N(0,1), constant coefficient row x5, eps 1e-7 (legacy_optim.py:187-213)
+        G = gen((512, 2048), 1235, 1.0)
+        fn = lambda: H.zeropower_via_newtonschulz5_legacy(G, steps=5)
+        ms = _time_calls(fn, 200, warm=5)
+        out["config1"] = pack(ms, [((512, 2048), 1)], _instrumented(fn),
+                              workload="NS5 of one 512x2048 matrix, constant coefficients, half-precision workspace")
+    if 3 in which:   # 64 experts: stacked W1/W3 512x2048 and W2 2048x256, full MuonH step with per-expert norms
+        ms, recs, n = muonh_step_config([(64, 512, 2048), (64, 2048, 256)], 1237, 100)
+        out["config3"] = pack(ms, [((512, 2048), 64), ((2048, 256), 64)], recs, elements=n,
+                              workload="full MuonH step, (64,512,2048) + (64,2048,256) expert stacks")
+        _lib.release_workspaces()
+    if 4 in which:   # NS5 of one large heavy-tailed matrix (Student-t df=3, std 1e-3, 1 % of the rows zeroed)
+        for name, shape, seed in (("config4_8192x8192", (8192, 8192), 1239), ("config4_4096x14336", (4096, 14336), 1238)):
+            g = torch.Generator(device=dev).manual_seed(seed)
+            z = torch.randn(*shape, generator=g, device=dev)
+            chi = torch.randn(3, *shape, generator=g, device=dev).square().sum(0)
+            t = z / (chi / 3).sqrt() / (3.0 ** 0.5) * 1e-3
+            t[torch.randperm(shape[0], generator=g, device=dev)[: shape[0] // 100]] = 0
+            G = t.to(torch.bfloat16)
+            del z, chi, t
+            fn = lambda: H.zeropower_via_newtonschulz5(G, 1e-7)
+            ms = _time_calls(fn, 10)
+            out[name] = pack(ms, [(shape, 1)], _instrumented(fn), workload=f"NS5 of one {shape[0]}x{shape[1]} matrix, "
+                             "production coefficients")
+            del G
+            _lib.release_workspaces()
+            torch.cuda.empty_cache()
+    if 5 in which and torch.cuda.mem_get_info(dev)[0] > (150 << 30):
+        layer = [(3072, 3072), (768, 3072), (768, 3072), (3072, 3072), (1536, 3072), (1536, 3072), (3072, 1536),
+                 (64, 768, 3072), (64, 3072, 384)]
+        torch.cuda.reset_peak_memory_stats(dev)
+        ms, recs, n = muonh_step_config(layer * 24, 1240, 5)
+        counts = [((3072, 3072), 48), ((768, 3072), 48 + 24 * 64), ((1536, 3072), 72), ((3072, 384), 24 * 64)]
+        out["config5"] = pack(ms, counts, recs, elements=n,
+                              peak_hbm_allocated_gib=round(torch.cuda.max_memory_allocated(dev) / 2 ** 30, 1),
+                              workload="full MuonH step, depth-24 MoE set (6.34 G elements, 64 routed experts per layer)")
+        _lib.release_workspaces()
+        torch.cuda.empty_cache()
+    return out
+
+
+TRAFFIC_PROFILE = "profiles/bench_config2_ns_gemm_and_epilogues.md"
+
+
 def measured_traffic(kernel_name):
     """HBM bytes per launch of `kernel_name` from the committed counter summary (two `rocprofv3 --pmc` runs,
     FETCH_SIZE and WRITE_SIZE, each scaled by the reading of a plain copy of known size), or None."""
-    path = os.path.join(ROOT, "profiles", "bench_config2_ns_gemm_and_epilogues.md")
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
     try:
         for line in open(path):
             line = line.strip()
@@ -113,6 +218,10 @@ def main():
     ap.add_argument("--separate-momentum", action="store_true",
                     help="(comparison) momentum kernel and Newton-Schulz as separate library calls instead of the fused one")
     ap.add_argument("--seed", type=int, default=1236)
+    ap.add_argument("--min-timed-seconds", type=float, default=2.0,
+                    help="the block of --steps steps is repeated until the timed region is at least this long")
+    ap.add_argument("--other-configs", default="1,3,4,5",
+                    help="comma-separated benchmark configurations reported beside the headline (empty: none)")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain device copy run once after the steps (yardstick for HBM byte counters)")
     args = ap.parse_args()
@@ -139,12 +248,19 @@ def main():
     for _ in range(args.warmup):  # also warms the momentum so that M != G
         opt.step()
     torch.cuda.synchronize()
+    # the timed region: blocks of exactly --steps steps, repeated (whole blocks only) until at least
+    # --min-timed-seconds have passed; ms_per_step is the mean over every timed step
+    repeats, wall = 0, 0.0
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        opt.step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
+    while True:
+        for _ in range(args.steps):
+            opt.step()
+        torch.cuda.synchronize()
+        repeats += 1
+        wall = time.perf_counter() - t0
+        if wall >= args.min_timed_seconds or repeats >= 1000:
+            break
+    ms_per_step = wall / (args.steps * repeats) * 1e3
 
     # one more, instrumented step: HIP events around every phase and every Newton-Schulz GEMM launch
     opt.phase_events = []
@@ -175,6 +291,8 @@ def main():
 
     # dominant kernel: the X' = aX + BX product in its main (non-final) instantiation
     by_kernel = {}
+    mom = [r for r in recs if r["kind"] == "momentum_layout"]
+    recs = [r for r in recs if r["kind"] == "gemm"]
     for r in recs:
         k = (r["tile"], r["mode"], r["split"], r["final"], r["folded"])
         d = by_kernel.setdefault(k, dict(n=0, ms=0.0, fa=0.0, fi=0.0))
@@ -203,6 +321,9 @@ def main():
     }
     if args.layers == N_LAYERS:
         roofline["traffic"] = measured_traffic(roofline["kernel"])
+        # not measured in this run: counters need rocprofv3 passes of their own
+        roofline["traffic_source"] = (f"{TRAFFIC_PROFILE} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
+                                      "scaled by the calibration copy; committed summary, not measured in this run)")
     if dom_key[1] == 2:  # B (m^2), X^T read (once more as the addend unless a*I is folded into B), X'^T written: bf16
         reads_x = 1 if dom_key[4] else 2
         per = [(min(s) ** 2 + (reads_x + 1) * min(s) * max(s)) * 2.0 for s in shapes]
@@ -216,6 +337,21 @@ def main():
             gbs = n_elem * bytes_per_elem[name] / ms / 1e6
             hbm[name] = {"ms": round(ms, 3), "GB/s": round(gbs, 0), "frac": round(gbs / HBM_PEAK_GBS, 3),
                          "bytes_per_elem": bytes_per_elem[name]}
+    if mom:   # fused momentum + layout launches (one per shape class), timed per launch inside the library call
+        mms, mbytes = sum(r["ms"] for r in mom), sum(r["bytes"] for r in mom)
+        hbm["momentum_layout"] = {"ms": round(mms, 3), "GB/s": round(mbytes / mms / 1e6, 0),
+                                  "frac": round(mbytes / mms / 1e6 / HBM_PEAK_GBS, 3), "bytes_per_elem": 8.0,
+                                  "launches": len(mom)}
+    # per-product share of the bf16 matrix-core peak (issued / algorithmic FLOPs over the summed launch durations)
+    kernel_fracs = {}
+    for label, modes in (("syrkt", (0, 3)), ("syrk2", (1,)), ("bx", (2,))):
+        sel = [r for r in recs if r["mode"] in modes]
+        if sel:
+            t = sum(r["ms"] for r in sel)
+            kernel_fracs[label] = {
+                "issued_frac": round(sum(r["flops_issued"] for r in sel) / t / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "algorithmic_frac": round(sum(r["flops_algorithmic"] for r in sel) / t / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "ms_per_step": round(t, 3)}
     ns_ms = sum(ms for n, ms in phases.items() if n.startswith("newton_schulz"))  # norms, layout and the 15 grouped GEMMs
 
     out = {
@@ -224,6 +360,7 @@ def main():
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3),
+        "timed_repeats": repeats, "timed_region_s": round(wall, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if args.precision == "f16" else "bf16", "data": "synthetic",
         "config": {"workload": f"config 2: full MuonH step, depth-{args.layers} GQA transformer, "
@@ -236,11 +373,19 @@ def main():
         "ns_gemm_pct_mfma_peak_symmetric": round(f_sym / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
         "ns_gemm_ms": round(gemm_ms, 3), "ns_phase_ms": round(ns_ms, 3),
         "roofline": roofline,
+        "kernel_fracs": kernel_fracs,
         "kernels": kernels,
         "hbm_kernels": hbm,
         "phases_ms": {k: round(v, 3) for k, v in phases.items()},
         "calibration_copy_bytes": cal_bytes,
     }
+    which = [int(x) for x in args.other_configs.split(",") if x.strip()]
+    if which and args.layers == N_LAYERS:
+        # the headline's tensors are released first (config 5 needs 80 GiB of its own)
+        del opt, params, grads, p, g
+        _lib.release_workspaces()
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(dev, which)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.coeffs, args.seed)
     print(json.dumps(out))

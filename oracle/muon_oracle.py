@@ -247,6 +247,53 @@ def msign(G: Tensor, steps: int, *, storage: str = "bf16_eager") -> Tensor:
     return X.contiguous()
 
 
+def emerging_newton_schulz(x: Tensor, steps: int, coefficient_type: str = "polar_express",
+                           custom_coefficient_sets: Optional[Coeffs] = None, eps: float = 1e-7,
+                           transpose: Optional[bool] = None, *, storage: str = "bf16_eager") -> Tensor:
+    """emerging_optimizers/orthogonalized_optimizers/muon_utils.py:68-164: fp32 input required; transpose (given, or
+    rows > cols); F.normalize over the last two dimensions in fp32 (X / max(|X|, eps), :125); named coefficient set or
+    a custom one, ``steps`` a multiple of its length and the set cycled ``i % len(set)`` (:127-139, :157-158); the
+    normalised matrix rounded to bf16 (:144) and iterated with newton_schulz_step_tsyrk (:262-287: A = XX^T,
+    B = cAA + bA, X' = BX + aX, each a bf16 product); fp32 result, transposed back.
+
+    storage "bf16_eager": every product rounds to bf16 (the reference's semantics);
+            "fp32": the same rounded input iterated in fp32 (tolerance oracle)."""
+    if x.ndim < 2:
+        raise ValueError("Input tensor x must have at least 2 dimensions since Muon is not for 1d parameters.")
+    if x.dtype != torch.float32:
+        raise ValueError(f"Input tensor x must be in float32, got {x.dtype}")
+    if transpose is None:
+        transpose = x.size(-2) > x.size(-1)
+    if transpose:
+        x = x.mT
+    X = x / x.norm(dim=(-2, -1), keepdim=True).clamp_min(eps)
+    named = {"simple": SIMPLE, "quintic": QUINTIC, "polar_express": POLAR_EXPRESS, "aol": AOL}
+    if coefficient_type in named:
+        sets = named[coefficient_type]
+    elif coefficient_type == "custom":
+        if custom_coefficient_sets is None:
+            raise ValueError("custom_coefficient_sets must be provided when coefficient_type is 'custom'.")
+        sets = custom_coefficient_sets
+    else:
+        raise ValueError(f"Invalid coefficient type: {coefficient_type}")
+    if steps % len(sets) != 0:
+        raise ValueError(f"steps ({steps}) must be multiple of len(coefficient_sets) ({len(sets)}).")
+    X = X.to(torch.bfloat16)
+    if storage == "fp32":
+        X = X.to(torch.float32)
+    elif storage != "bf16_eager":
+        raise ValueError(storage)
+    for i in range(steps):
+        a, b, c = sets[i % len(sets)]
+        A = X @ X.mT
+        B = c * (A @ A) + b * A
+        X = B @ X + a * X
+    X = X.to(torch.float32)
+    if transpose:
+        X = X.mT
+    return X.contiguous()
+
+
 def ns_singular_value_map(s: Tensor, coeffs: Coeffs) -> Tensor:
     """Scalar action of the iteration on one singular value: p(s) = a s + b s^3 + c s^5
     applied once per row of ``coeffs`` (what NS does in exact arithmetic)."""

@@ -201,16 +201,27 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             found |= set(range(int(a), int(b) + 1)) if a else {int(c)}
         return found
 
-    kernels = reads = 0
-    pending, inside, in_asm = set(), False, False
+    # template arguments of an instantiation from its mangled name: <BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>
+    targs = re.compile(r"ns_gemm_kernelILi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])ELb([01])ELi(\d+)EE")
+    seen, reads_of = set(), {}
+    all_kernels = 0
+    pending, inside, in_asm, cur = set(), False, False, None
     for line in text:
         if "#ASMSTART" in line or "#ASMEND" in line:
             in_asm = "#ASMSTART" in line
             continue
         code = line.split(";")[0].strip()
         if code.endswith(":") and "ns_gemm_kernel" in code:
-            inside = "ELi3ELb" in code          # MODE_SYRKT instantiations
-            kernels += inside
+            m = targs.search(code)
+            assert m, f"cannot read the template arguments of {code}: the name mangling changed, adapt this test"
+            all_kernels += 1
+            bm, mode, f16 = int(m.group(1)), int(m.group(5)), int(m.group(9))
+            inside = mode == 3                   # MODE_SYRKT instantiations
+            cur = (bm, f16)
+            if inside:
+                assert cur not in seen, f"{code} seen twice"
+                seen.add(cur)
+                reads_of[cur] = 0
             pending = set()
             continue
         if not inside or not code or code.startswith("."):
@@ -224,10 +235,15 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             assert not (regs(addr) & pending), line
             assert not (regs(dst) & pending), line
             pending |= regs(dst)
-            reads += 1
+            reads_of[cur] += 1
             continue
         if code.startswith("s_waitcnt") and "lgkmcnt(0)" in code:
             pending = set()
             continue
         assert not (regs(code) & pending), f"uses a transpose-read result before the wait: {line}"
-    assert kernels == 4 and reads >= 4 * 12 * 4      # two tile configurations x {bfloat16, half} workspace
+    # every K-major instantiation was visited by name: two tile configurations x {bfloat16, half} workspace
+    assert seen == {(256, 0), (256, 1), (128, 0), (128, 1)}, seen
+    assert all_kernels > len(seen)
+    # per k-tile: 4 k-steps x (FM + FN) fragments x 2 reads; the loop body appears at least once
+    assert all(reads_of[(256, f)] >= 4 * 6 * 2 for f in (0, 1)), reads_of
+    assert all(reads_of[(128, f)] >= 4 * 4 * 2 for f in (0, 1)), reads_of

@@ -42,7 +42,8 @@ def test_config2_full_step(gpu_device):
     for p, gr in zip(params, grads):
         p.grad = gr
     opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, use_muonh=True)
-    sample = [1, 6, 4, 59, 111]  # a Wk, a W2 (wide), a W1 (tall), and two more
+    # every kind of matrix of a layer (Wq, Wk, Wv, Wo, W1, W3, W2), early, middle and late layers
+    sample = [0, 1, 6, 4, 2 * 7 + 5, 7 * 7 + 3, 8 * 7 + 3, 59, 12 * 7 + 2, 15 * 7 + 0, 15 * 7 + 5, 111]
     w0 = {i: params[i].detach().cpu().clone() for i in sample}
     norms0 = torch.stack([p.detach().float().norm() for p in params])
     # two steps, so that the second one runs with momentum != gradient
@@ -89,10 +90,9 @@ def test_config4_large_heavy_tailed(gpu_device, shape, seed, table):
     got = got.cpu()
     assert torch.all(got[zero_rows] == 0)
     assert torch.isfinite(got.float()).all()
-    if shape == (4096, 14336) or table == "quintic":
-        # full fp32 oracle on the host (seconds for 4096x14336, under a minute for 8192^2)
-        want = O.newton_schulz(G, coeffs, 1e-7, storage="fp32")
-        assert _rel(got, want) <= NS_TOL
+    # full fp32 oracle on the host (seconds for 4096x14336, under a minute for 8192^2)
+    want = O.newton_schulz(G, coeffs, 1e-7, storage="fp32")
+    assert _rel(got, want) <= NS_TOL
     # squared row norms are the diagonal of O O^T = U p(S)^2 U^T: bounded by the square of the band's upper end,
     # and their sum is the number of singular values pushed to ~1 (the rank, here the non-zero rows)
     sq = got.float().square().sum(dim=1)

@@ -404,3 +404,29 @@ def test_half_precision_workspace_scales(ns, gpu_device):
     sv = torch.linalg.svdvals(got[:, :4096].float().cpu() @ got[:, :4096].float().cpu().T + got[:, 4096:].float().cpu() @ got[:, 4096:].float().cpu().T)
     # singular values of the result squared: the production schedule lands every one of them in (0.4, 1.3)^2
     assert sv.min().item() > 0.16 and sv.max().item() < 1.7
+
+
+@pytest.mark.parametrize("kind,steps", [("simple", 5), ("quintic", 5), ("quintic", 10), ("polar_express", 8),
+                                        ("polar_express", 16), ("aol", 4), ("aol", 8), ("custom", 4)])
+@pytest.mark.parametrize("shape", [(320, 1100), (1100, 320), (257, 257), (3, 200, 136)])
+def test_emerging_newton_schulz_named_sets(gpu_device, kind, steps, shape):
+    """emerging_optimizers' newton_schulz (fp32 in, fp32 out, clamp eps, named sets cycled) through the HIP path against
+    the oracle's restatement iterated in fp32 on the same rounded input."""
+    from archscale_amd.emerging.muon_utils import newton_schulz
+    print("case", kind, steps, shape, flush=True)
+    g = torch.Generator().manual_seed(17 + steps + sum(shape))
+    x = torch.randn(*shape, generator=g) * 3e-2
+    custom = [(3.0, -3.2, 1.2), (2.0, -1.5, 0.5)] if kind == "custom" else None
+    got = newton_schulz(x.to(gpu_device), steps, kind, custom)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.float32 and got.shape == x.shape
+    want = O.emerging_newton_schulz(x, steps, kind, custom, storage="fp32")
+    err = _rel(got, want)
+    print("rel err", err, flush=True)
+    assert err <= NS_TOL
+    # no further from the fp32 run than the reference's own all-bf16 arithmetic is
+    eager = O.emerging_newton_schulz(x, steps, kind, custom)
+    assert err <= max(_rel(eager, want), 4e-3)
+    # an explicit transpose flag (either value) changes nothing
+    flipped = newton_schulz(x.to(gpu_device), steps, kind, custom, transpose=shape[-2] <= shape[-1])
+    assert torch.equal(flipped, got)

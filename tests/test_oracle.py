@@ -35,6 +35,48 @@ def test_ns_fp32_matches_svd_closed_form(shape, table):
     assert (got - want).norm() / want.norm() < 2e-4
 
 
+@pytest.mark.parametrize("kind,steps", [("simple", 3), ("quintic", 5), ("polar_express", 8), ("aol", 4), ("aol", 8),
+                                        ("custom", 4)])
+@pytest.mark.parametrize("shape", [(20, 48), (48, 20)])
+def test_emerging_newton_schulz_matches_svd_closed_form(kind, steps, shape):
+    """fp32 in / fp32 out, clamp eps, the named set cycled: against U diag(p(s / max(|X|, eps))) V^T from an fp64 SVD of
+    the bf16-rounded normalised input (a wrong table row, a set indexed without the modulo or eps added instead of
+    clamped fails this)."""
+    g = torch.Generator().manual_seed(sum(shape) + steps)
+    x = torch.randn(*shape, generator=g)
+    custom = [(3.0, -3.2, 1.2), (2.0, -1.5, 0.5)] if kind == "custom" else None
+    sets = {"simple": O.SIMPLE, "quintic": O.QUINTIC, "polar_express": O.POLAR_EXPRESS, "aol": O.AOL, "custom": custom}[kind]
+    rows = [sets[i % len(sets)] for i in range(steps)]
+    xn = (x / x.norm().clamp_min(1e-7)).to(torch.bfloat16).to(torch.float64)
+    U, S, Vh = torch.linalg.svd(xn, full_matrices=False)
+    want = U @ torch.diag_embed(O.ns_singular_value_map(S, rows)) @ Vh
+    got = O.emerging_newton_schulz(x, steps, kind, custom, storage="fp32")
+    assert got.dtype == torch.float32 and got.shape == x.shape
+    assert (got.double() - want).norm() / want.norm() < 5e-4
+    # the reference's own (all-bf16) semantics stay close to it; an explicit transpose flag changes nothing mathematically
+    eager = O.emerging_newton_schulz(x, steps, kind, custom)
+    assert (eager.double() - want).norm() / want.norm() < 6e-2
+    flipped = O.emerging_newton_schulz(x, steps, kind, custom, transpose=shape[0] <= shape[1], storage="fp32")
+    assert (flipped.double() - want).norm() / want.norm() < 5e-4
+    # eps is a clamp, not an addend: a huge eps divides by eps exactly
+    big = O.emerging_newton_schulz(x, 1, "custom", [(1.0, 0.0, 0.0)], eps=1e3, storage="fp32")
+    assert torch.allclose(big, (x / 1e3).to(torch.bfloat16).float(), rtol=1e-6, atol=0)
+
+
+def test_emerging_newton_schulz_errors():
+    x = torch.randn(4, 8)
+    with pytest.raises(ValueError):
+        O.emerging_newton_schulz(x, 5, "aol")                 # 5 is no multiple of 4
+    with pytest.raises(ValueError):
+        O.emerging_newton_schulz(x.double(), 5, "quintic")
+    with pytest.raises(ValueError):
+        O.emerging_newton_schulz(x, 5, "custom")
+    with pytest.raises(ValueError):
+        O.emerging_newton_schulz(x, 5, "nope")
+    with pytest.raises(ValueError):
+        O.emerging_newton_schulz(torch.randn(8), 5, "quintic")
+
+
 def test_ns_singular_map_is_polynomial():
     # a plausible slip (dropping the s^5 term, or using s^2) must fail this
     s = torch.tensor([0.0, 0.1, 0.5, 1.0], dtype=torch.float64)
