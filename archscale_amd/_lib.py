@@ -25,6 +25,8 @@ NS_CAST_INPUT_FIRST = 1
 NS_NO_NORMALIZE = 2
 NS_NO_DIAG_FOLD = 4
 CHUNK_ELEMS = 8192
+NS_STATIC_SCRATCH_BYTES = 64 << 20
+E_STATIC_LIMIT = -4
 PROF_KEY_MOMENTUM_LAYOUT = 90000
 ABI_VERSION = 2
 
@@ -85,6 +87,12 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_ns_batched_static": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p]),
     "muon_ns_grouped_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(NsProblem), ctypes.c_int, ctypes.c_int]),
     "muon_ns_grouped": (ctypes.c_int, [
         ctypes.POINTER(NsProblem), ctypes.c_int,

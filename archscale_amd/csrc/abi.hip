@@ -171,6 +171,34 @@ hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const Grou
 
 }  // namespace
 
+// Scratch of muon_ns_batched_static: a device array that exists from the moment the code object is loaded, so that entry
+// point allocates nothing.  In host code this NAME is only a handle for hipGetSymbolAddress; kernels and copies get the
+// device address that the lookup returns (one per device: every GPU holds its own copy of the array).
+static __device__ __align__(256) unsigned char scratch[MUON_NS_STATIC_SCRATCH_BYTES];
+
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// device address of `scratch` on the CURRENT device (looked up once per device)
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return MUON_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr || ((uintptr_t)ptr & 255)) return MUON_E_WORKSPACE;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
 extern "C" {
 
 int muon_abi_version(void) { return MUON_ABI_VERSION; }
@@ -180,6 +208,8 @@ const char* muon_status_string(int status) {
   if (status == MUON_E_ARG) return "invalid argument (null pointer, non-positive extent or unknown enum)";
   if (status == MUON_E_WORKSPACE) return "workspace too small or not 256-byte aligned";
   if (status == MUON_E_UNSUPPORTED) return "unsupported configuration";
+  if (status == MUON_E_STATIC_LIMIT)
+    return "the problem needs more than MUON_NS_STATIC_SCRATCH_BYTES of workspace; call muon_ns_batched with a workspace of muon_ns_workspace_bytes()";
   if (status > 0) return hipGetErrorString((hipError_t)status);
   return "unknown status";
 }
@@ -529,6 +559,21 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
   q.batch = batch; q.rows = rows; q.cols = cols;
   if (!ws_dev) return MUON_E_ARG;
   return muon_ns_grouped(&q, 1, abc_host, iters, eps, eps_mode, prec_mode, flags, ws_dev, ws_bytes, stream);
+}
+
+int muon_ns_batched_static(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld, void* out_dev,
+                           int64_t out_batch_stride, int out_ld, int batch, int rows, int cols, const float* abc_host,
+                           int iters, float eps, int eps_mode, int prec_mode, int flags, void* stream) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return MUON_E_ARG;
+  if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT && prec_mode != MUON_PREC_F16) return MUON_E_ARG;
+  if (plan_bytes_bound(batch, rows, cols, prec_mode) > (size_t)MUON_NS_STATIC_SCRATCH_BYTES) return MUON_E_STATIC_LIMIT;
+  void* ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st) return st;
+  // every byte of the workspace that a kernel reads is written earlier in the same call (the layout pass writes the
+  // zero padding, the products write whole tiles), so nothing left over from the previous call has to be cleared
+  return muon_ns_batched(in_dev, in_dtype, in_batch_stride, in_ld, out_dev, out_batch_stride, out_ld, batch, rows, cols,
+                         abc_host, iters, eps, eps_mode, prec_mode, flags, ws, MUON_NS_STATIC_SCRATCH_BYTES, stream);
 }
 
 size_t muon_syrk_workspace_bytes(int batch, int n, int k) {

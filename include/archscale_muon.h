@@ -57,6 +57,7 @@ extern "C" {
 #define MUON_E_ARG (-1)        /* null pointer, non-positive extent, bad enum */
 #define MUON_E_WORKSPACE (-2)  /* workspace too small or misaligned */
 #define MUON_E_UNSUPPORTED (-3)
+#define MUON_E_STATIC_LIMIT (-4) /* muon_ns_batched_static: the problem needs more than MUON_NS_STATIC_SCRATCH_BYTES */
 
 /* elements covered by one block of the multi-tensor kernels; chunk prefixes are in these units */
 #define MUON_CHUNK_ELEMS 8192
@@ -89,6 +90,22 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
                     int batch, int rows, int cols,
                     const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
                     void* ws_dev, size_t ws_bytes, void* stream);
+
+/* muon_ns_batched for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * muon_ns_batched, without the workspace: the library's own scratch is a device array of
+ * MUON_NS_STATIC_SCRATCH_BYTES that is part of the loaded code object (every GPU the library runs on holds it until
+ * the process ends), and the call performs no hipMalloc / hipFree and calls no allocating library routine.
+ * A problem whose muon_ns_workspace_bytes(batch, rows, cols, prec_mode) exceeds MUON_NS_STATIC_SCRATCH_BYTES is
+ * rejected with MUON_E_STATIC_LIMIT before anything is launched.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered and safe.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside a capture. */
+#define MUON_NS_STATIC_SCRATCH_BYTES (64u << 20)
+int muon_ns_batched_static(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld,
+                           void* out_dev, int64_t out_batch_stride, int out_ld,
+                           int batch, int rows, int cols,
+                           const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
+                           void* stream);
 
 /* The same for several independent batches of different shapes at once (all shape classes of an optimizer
  * step): each product of the iteration is ONE kernel launch over the tiles of every problem, so there are
