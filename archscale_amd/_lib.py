@@ -24,6 +24,8 @@ SN_TRANSPOSED = 1
 NS_CAST_INPUT_FIRST = 1
 NS_NO_NORMALIZE = 2
 NS_NO_DIAG_FOLD = 4
+NS_NO_GRAM_TAIL = 8
+NS_GRAM_TAIL = 16
 CHUNK_ELEMS = 8192
 NS_STATIC_SCRATCH_BYTES = 64 << 20
 E_STATIC_LIMIT = -4

@@ -54,7 +54,10 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   p.cpm = (int)(((long)rows * cols + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = (size_t)round_up((long)(off + bytes), 256); return o; };
-  const size_t xb = (size_t)batch * p.Mp * p.Np * 2, ab = (size_t)batch * p.Mp * p.Mp * 2;
+  // a class whose long side is at least twice the short one may finish on the Gram side (see ns_grouped_impl): the idle
+  // X^T buffer then holds two more m x m matrices per matrix
+  const size_t ab = (size_t)batch * p.Mp * p.Mp * 2;
+  const size_t xb = std::max((size_t)batch * p.Mp * p.Np * 2, p.n >= 2 * p.m ? 2 * ab : (size_t)0);
   p.off_xt[0] = take(xb);
   p.off_xt[1] = take(xb);
   p.off_a = take(ab);
@@ -241,6 +244,7 @@ struct NsProblem {
   __bf16 *Xt[2], *A, *Bh, *Bl;   // Xt: the iterate as X^T, [b][Np][Mp] (long side first), ping-pong
   float *partial, *scale, *pow2;
   bool tall;
+  bool gram_tail;   // the last two iterations run on the Gram side (n >= 2m): one B X product instead of two
   bool defer;   // the operand of the first iteration is the input as it is; its epilogues apply 1/(|X| + eps)
   int sx;   // half-precision mode: the iterate is kept times 2^sx (its rms entry starts at about 2^-3)
 };
@@ -282,7 +286,10 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   const bool split_any = prec_mode == MUON_PREC_BF16_BSPLIT;
   const int split_tail = (flags >> 8) & 0xff;   // 0: every iteration keeps B as a hi+lo pair; t: only the last t
-  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | MUON_NS_NO_NORMALIZE | MUON_NS_NO_DIAG_FOLD | 0xff00)) return MUON_E_ARG;
+  if (flags & ~(MUON_NS_CAST_INPUT_FIRST | MUON_NS_NO_NORMALIZE | MUON_NS_NO_DIAG_FOLD | MUON_NS_NO_GRAM_TAIL |
+                MUON_NS_GRAM_TAIL | 0xff00))
+    return MUON_E_ARG;
+  if ((flags & MUON_NS_NO_GRAM_TAIL) && (flags & MUON_NS_GRAM_TAIL)) return MUON_E_ARG;
   const bool normalize = !(flags & MUON_NS_NO_NORMALIZE);
   if (!normalize && fused) return MUON_E_ARG;
   bool split = split_any;
@@ -325,11 +332,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     // second time is what a matrix with a few dominant singular values is sensitive to (Gaussian plus a 30x rank-one
     // spike, error against an fp32 run: 5.2e-2 -> 5.0e-3 in bfloat16, 6.7e-3 -> 1.8e-3 with the half workspace).
     P.defer = fused || (normalize && (P.q.in_dtype == MUON_DTYPE_BF16 || cast_first));
-    P.sx = 0;
-    if (f16) {
-      const int l2 = (int)floor(0.5 * log2((double)P.pl.m * (double)P.pl.n)) - 3;
-      P.sx = l2 > 0 ? l2 : 0;
-    }
+    const int l2 = (int)floor(0.5 * log2((double)P.pl.m * (double)P.pl.n)) - 3;
+    P.sx = l2 > 0 ? l2 : 0;   // used by the iterations that keep the iterate in half
+    P.gram_tail = false;
   }
   // the half workspace starts with a bfloat16 iteration when the scale is deferred (see the iteration below); one
   // kernel type per launch, so either every problem of the call defers or none does
@@ -399,15 +404,15 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     if (e != hipSuccess) return (int)e;
   }
 
-  // one product of the iteration for every problem: problems that share a tile configuration go into one
-  // launch (at most MAX_GROUPS per launch)
-  auto run_mode = [&](int mode, bool last, int ws16, auto&& fill) -> hipError_t {
+  // one product of the iteration for every problem that `fill` accepts: problems that share a tile configuration go
+  // into one launch (at most MAX_GROUPS per launch)
+  auto run_mode = [&](int mode, bool split_launch, bool final_, int ws16, auto&& fill) -> hipError_t {
     for (int tile : {256, 128}) {
       GroupedGemmParams gp = {};
       double fa = 0.0, fi = 0.0;
       auto flush = [&]() -> hipError_t {
         if (gp.n_groups == 0) return hipSuccess;
-        hipError_t err = launch_rounds(tile, mode, split && (mode == MODE_SYRK2 || mode == MODE_BX), last && mode == MODE_BX, gp, stream, fa, fi, ws16);
+        hipError_t err = launch_rounds(tile, mode, split_launch, final_, gp, stream, fa, fi, ws16);
         gp = GroupedGemmParams{};
         fa = fi = 0.0;
         return err;
@@ -417,7 +422,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
         if (P.pl.tile != tile) continue;
         GemmParams g = {};
         double a_fl = 0.0, i_fl = 0.0;
-        fill(P, g, a_fl, i_fl);
+        if (!fill(P, g, a_fl, i_fl)) continue;
         const long tiles = ns_gemm_tiles(mode, g);
         if (tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L || gp.n_groups == MAX_GROUPS) {
           hipError_t err = flush();
@@ -436,72 +441,139 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     return hipSuccess;
   };
 
-  int cur = 0;
-  for (int it = 0; it < iters; ++it) {
-    const float a = abc_host[3 * it], b = abc_host[3 * it + 1], c = abc_host[3 * it + 2];
-    const bool last = it == iters - 1;
-    split = split_any && (split_tail == 0 || it >= iters - split_tail);
+  // ---- storage of the iteration's matrices, per iteration.  MUON_PREC_F16: half from the first iteration on, or from
+  // the second one when the scale is deferred - the unnormalised operand cannot go into half as it is (its magnitude is
+  // the gradient's), so the first iteration then runs on it in bfloat16 with the deferred scale and its last product
+  // writes X' as scaled half; the operand of that iteration is the exact bfloat16 update, and A and B of ONE early
+  // iteration in bfloat16 cost nothing measurable (error against an fp32 run, CPU model, 512x2048 / 1024x1024 / 64x129:
+  // constant row 2.15 / 2.01 / 2.27e-3 against 2.16 / 2.03 / 2.22e-3 with all five in half; a second bfloat16 iteration
+  // would cost 3.3 / 3.7 / 9.2e-3).
+  // MUON_PREC_BF16 with at least three iterations: the LAST TWO iterations run in half as well ("tail").  Their
+  // matrices are bounded whatever the input was, the rounding of the last iterations dominates the error of the result
+  // (CPU model, quintic schedule, error against an fp64 run: Gaussian 4.5e-3 -> 3.3e-3, 300x rank-one spike
+  // 1.9e-2 -> 1.6e-2), and half is what makes the Gram-side tail below as accurate as the iteration on X.
+  auto fold_ok = [&](int it) {
+    return !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(abc_host[3 * it]) <= 4.2f;
+  };
+  // (an input that is not normalised is not bounded: no half storage that the caller did not ask for)
+  // On by default under MUON_PREC_BF16, where it lowers the error on every spectrum tried; under MUON_PREC_F16 it costs
+  // 1-2 % of accuracy (polar-express msign table, whose spectrum is not settled two iterations before the end:
+  // 1.9e-3 -> 2.4e-3), so there the caller has to ask for it.
+  const bool tail_wanted = (flags & MUON_NS_NO_GRAM_TAIL) ? false : ((flags & MUON_NS_GRAM_TAIL) ? true : !f16);
+  const bool tail = tail_wanted && normalize && !split_any && iters >= 3 && fold_ok(iters - 2) && fold_ok(iters - 1);
+  const int first_half_it = f16 ? (defer_all ? 1 : 0) : (tail ? iters - 2 : iters);
+  // ---- Gram-side tail.  With P_k = a_k I + b_k A_k + c_k A_k^2 (symmetric, a polynomial in A_k = X_k X_k^T, so all of
+  // them commute) the last two iterations are  X_N = P_N P_{N-1} X_{N-2}  with  A_{N-1} = P_{N-1} A_{N-2} P_{N-1}:
+  // three more m x m symmetric products (T = P A, A' = T P, Q = P' P) replace one B X and one X X^T product, which
+  // saves 3 m^2 (n - m) multiply-adds per matrix - 11 % of a 2048 x 5632 matrix's iteration.  Taken for the classes
+  // with n >= 2m.  Only the LAST two iterations: earlier, the spectrum still spans orders of magnitude and squaring it
+  // pushes the small singular values under the rounding of the Gram matrix (CPU model, fusing three iterations:
+  // log-spaced spectrum 3e-2 -> 1.6e-1).  With the tail in half the result is as close to an fp64 run as the iteration
+  // on X (Gaussian 3.26e-3 / 3.28e-3, 300x spike 1.62e-2 / 1.62e-2, log-spaced spectrum 3.00e-2 / 3.01e-2, low rank
+  // plus noise 4.54e-2 / 4.54e-2 without / with it; MUON_PREC_F16: 1.74 / 1.77e-3, 3.9 / 4.0e-3, 4.2 / 4.5e-3, 7.2 / 7.3e-3).
+  bool any_tail = false, all_tail = true;
+  for (NsProblem& P : pr) {
+    P.gram_tail = tail && P.pl.n >= 2 * P.pl.m;
+    any_tail = any_tail || P.gram_tail;
+    all_tail = all_tail && P.gram_tail;
+  }
+  const int SH_A = 8, SH_B = 6;   // powers of two carried by A and by B, T, Q in half storage
+
+  struct ItCfg { float a, b, c; bool last, half_ops, half_out, fold, split; int SAi, SBi, ws16, bx16; };
+  auto it_cfg = [&](int it) {
+    ItCfg k;
+    k.a = abc_host[3 * it]; k.b = abc_host[3 * it + 1]; k.c = abc_host[3 * it + 2];
+    k.last = it == iters - 1;
+    k.half_ops = it >= first_half_it;
+    k.half_out = !k.last && it + 1 >= first_half_it;
+    k.split = split_any && (split_tail == 0 || it >= iters - split_tail);
     // a*I folded into B (diagonal entries of B + aI are rounded like any other entry): X' = (B + aI) X needs no addend.
     // Not for a large `a` (first row of the polar-express table), whose rounding on the diagonal would show, and not in
     // the first iteration: a matrix with a few dominant singular values has a tiny A after the normalisation, and
-    // B_ii would vanish below half an ulp of `a`.
-    // With the hi+lo pair the folded diagonal is exact; an iteration of a split call that keeps B in plain bf16 is not
-    // folded (constant coefficients on small matrices: 8.4e-3 -> 1.1e-2 for 64x129 when it is).
-    const bool fold = !(flags & MUON_NS_NO_DIAG_FOLD) && it > 0 && fabsf(a) <= 4.2f && (!split_any || split);
-    // Half-precision workspace with a deferred scale (after the fused momentum, or a bfloat16 input): the unnormalised
-    // operand cannot go into half as it is (its magnitude is the gradient's), so the first iteration runs on it in
-    // bfloat16 with the deferred scale, as in MUON_PREC_BF16, and its last product writes X' as scaled half.  The operand of that iteration is then the exact
-    // bfloat16 update, and A and B of ONE early iteration in bfloat16 cost nothing measurable (error against an fp32
-    // run, CPU model, 512x2048 / 1024x1024 / 64x129: constant row 2.15 / 2.01 / 2.27e-3 against 2.16 / 2.03 / 2.22e-3
-    // with all five iterations in half; a second bfloat16 iteration would cost 3.3 / 3.7 / 9.2e-3).
-    const bool lowp = f16 && defer_all && it == 0;
-    const int SAi = lowp ? 0 : SA, SBi = lowp ? 0 : SB;
-    const int ws16 = lowp ? 0 : (f16 ? 1 : 0);
-    // A = X X^T, from X^T (K-major operand)
-    e = run_mode(MODE_SYRKT, last, ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+    // B_ii would vanish below half an ulp of `a`.  With the hi+lo pair the folded diagonal is exact; an iteration of a
+    // split call that keeps B in plain bf16 is not folded (constant coefficients on small matrices: 8.4e-3 -> 1.1e-2
+    // for 64x129 when it is).
+    k.fold = fold_ok(it) && (!split_any || k.split);
+    k.SAi = k.half_ops ? SH_A : 0;
+    k.SBi = k.half_ops ? SH_B : 0;
+    k.ws16 = k.half_ops ? 1 : 0;
+    k.bx16 = k.half_ops ? 1 : (k.half_out ? 2 : 0);   // 2: bfloat16 operands, the next iterate in half
+    return k;
+  };
+  // A = X X^T of the iterate in Xt[src], from X^T (K-major operand)
+  auto syrkt = [&](int it, int src, auto&& want) -> hipError_t {
+    const ItCfg k = it_cfg(it);
+    return run_mode(MODE_SYRKT, false, false, k.ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      if (!want(P)) return false;
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
-      g.P = P.Xt[cur]; g.Q = P.Xt[cur]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
+      g.P = P.Xt[src]; g.Q = P.Xt[src]; g.strideP = g.strideQ = xs; g.ldp = g.ldq = pl.Mp; g.K = pl.Np;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
-      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, SAi - 2 * (lowp ? 0 : P.sx)); g.beta = 0.f;
+      g.C = P.A; g.strideC = as; g.ldc = pl.Mp; g.alpha = ldexpf(1.f, k.SAi - 2 * (k.half_ops ? P.sx : 0)); g.beta = 0.f;
       g.scale = (P.defer && it == 0) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
+      return true;
     });
-    if (e != hipSuccess) return (int)e;
-    // B = c A A + b A
-    e = run_mode(MODE_SYRK2, last, ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+  };
+  // B = c A A + b A (+ a I) into dst(P) (and the low half of the pair into P.Bl)
+  auto syrk2 = [&](int it, auto&& want, auto&& dst) -> hipError_t {
+    const ItCfg k = it_cfg(it);
+    return run_mode(MODE_SYRK2, k.split, false, k.ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      if (!want(P)) return false;
       const NsPlan& pl = P.pl;
       const long as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
       g.P = P.A; g.Q = P.A; g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
       g.tilesM = g.tilesN = pl.Mp / pl.tile;
       g.E = P.A; g.strideE = as; g.lde = pl.Mp;
-      g.C = P.Bh; g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp;
-      g.alpha = ldexpf(c, SBi - 2 * SAi); g.beta = ldexpf(b, SBi - SAi);
-      g.diag_add = fold ? ldexpf(a, SBi) : 0.f;
+      g.C = dst(P); g.C2 = P.Bl; g.strideC = as; g.ldc = pl.Mp;
+      g.alpha = ldexpf(k.c, k.SBi - 2 * k.SAi); g.beta = ldexpf(k.b, k.SBi - k.SAi);
+      g.diag_add = k.fold ? ldexpf(k.a, k.SBi) : 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
       fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
+      return true;
     });
-    if (e != hipSuccess) return (int)e;
-    // X' = a X + B X
-    e = run_mode(MODE_BX, last, (lowp && !last) ? 2 : ws16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+  };
+  // symmetric product of two symmetric m x m matrices in half storage: dst = 2^shift * L * R (upper triangle computed
+  // and mirrored; L and R commute)
+  auto symprod = [&](auto&& want, auto&& lhs, auto&& rhs, auto&& dst, int shift) -> hipError_t {
+    return run_mode(MODE_SYRK, false, false, 1, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      if (!want(P)) return false;
+      const NsPlan& pl = P.pl;
+      const long as = (long)pl.Mp * pl.Mp;
+      g.batch = P.q.batch;
+      g.P = lhs(P); g.Q = rhs(P); g.strideP = g.strideQ = as; g.ldp = g.ldq = pl.Mp; g.K = pl.Mp;
+      g.tilesM = g.tilesN = pl.Mp / pl.tile;
+      g.C = dst(P); g.strideC = as; g.ldc = pl.Mp;
+      g.alpha = ldexpf(1.f, shift); g.beta = 0.f;
+      const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
+      fa = bm * dm * dm * dm;
+      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
+      return true;
+    });
+  };
+  // X' = a X + B X with B = lhs(P) and X^T in Xt[src]; the next iterate goes to Xt[src ^ 1], the last one to the caller
+  auto bx = [&](int it, int src, auto&& want, auto&& lhs) -> hipError_t {
+    const ItCfg k = it_cfg(it);
+    return run_mode(MODE_BX, k.split, k.last, k.bx16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
+      if (!want(P)) return false;
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
-      g.P = P.Bh; g.P2 = P.Bl; g.Q = P.Xt[cur]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp;
+      g.P = lhs(P); g.P2 = P.Bl; g.Q = P.Xt[src]; g.strideP = as; g.strideQ = xs; g.ldp = pl.Mp; g.ldq = pl.Mp;
       g.K = pl.Mp;
       g.tilesM = pl.Mp / pl.tile; g.tilesN = pl.Np / pl.tile;
-      g.E = fold ? nullptr : P.Xt[cur]; g.strideE = xs; g.lde = pl.Mp;
-      g.alpha = ldexpf(a, SBi); g.beta = 0.f;
-      // the operand carries 2^sx (not in the bfloat16 iteration), the next iterate does, the caller's result does not
-      g.out_shift = -SBi - (lowp ? 0 : P.sx) + ((last || !f16) ? 0 : P.sx);
+      g.E = k.fold ? nullptr : P.Xt[src]; g.strideE = xs; g.lde = pl.Mp;
+      g.alpha = ldexpf(k.a, k.SBi); g.beta = 0.f;
+      // B carries 2^SB, a half operand 2^sx, a half result 2^sx; the caller's result carries nothing
+      g.out_shift = -k.SBi - (k.half_ops ? P.sx : 0) + (k.half_out ? P.sx : 0);
       g.scale = (P.defer && it == 0) ? P.scale : nullptr;
-      if (!last) {
-        g.Ct = P.Xt[cur ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
+      if (!k.last) {
+        g.Ct = P.Xt[src ^ 1]; g.strideCt = xs; g.ldct = pl.Mp;   // only X'^T: no product reads a row-major X
       } else {
         g.m_valid = pl.m; g.n_valid = pl.n;
         if (!P.tall) { g.C = (__bf16*)P.q.out; g.strideC = P.q.out_batch_stride; g.ldc = P.q.out_ld; }
@@ -509,10 +581,41 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       }
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * 2.0 * dm * dm * dn;
-      fi = bm * 2.0 * tl * tl * (double)(pl.Mp / pl.tile) * (pl.Np / pl.tile) * pl.Mp * (split ? 2.0 : 1.0);
+      fi = bm * 2.0 * tl * tl * (double)(pl.Mp / pl.tile) * (pl.Np / pl.tile) * pl.Mp * (k.split ? 2.0 : 1.0);
+      return true;
     });
-    if (e != hipSuccess) return (int)e;
+  };
+  auto every = [](const NsProblem&) { return true; };
+  auto on_gram = [](const NsProblem& P) { return P.gram_tail; };
+  auto plain = [](const NsProblem& P) { return !P.gram_tail; };
+  auto in_bh = [](const NsProblem& P) { return P.Bh; };
+
+  int cur = 0;
+  const int n_plain_iters = any_tail ? iters - 2 : iters;
+  for (int it = 0; it < n_plain_iters; ++it) {
+    if ((e = syrkt(it, cur, every)) != hipSuccess) return (int)e;
+    if ((e = syrk2(it, every, in_bh)) != hipSuccess) return (int)e;
+    if ((e = bx(it, cur, every, in_bh)) != hipSuccess) return (int)e;
     cur ^= 1;
+  }
+  if (any_tail) {
+    // X_{N-2} is in Xt[cur] (half); the idle buffer Xt[cur ^ 1] of a fused problem holds T / Q and P_N
+    const int i1 = iters - 2, i2 = iters - 1;
+    auto buf_t = [&](const NsProblem& P) { return P.Xt[cur ^ 1]; };
+    auto buf_p2 = [&](const NsProblem& P) { return P.Xt[cur ^ 1] + (size_t)P.q.batch * P.pl.Mp * P.pl.Mp; };
+    auto in_a = [](const NsProblem& P) { return P.A; };
+    if ((e = syrkt(i1, cur, every)) != hipSuccess) return (int)e;                                  // A1 = X X^T
+    if ((e = syrk2(i1, every, in_bh)) != hipSuccess) return (int)e;                                // P1 (in Bh)
+    if ((e = symprod(on_gram, in_bh, in_a, buf_t, SH_B - SH_B - SH_A)) != hipSuccess) return (int)e;  // T = P1 A1
+    if (!all_tail && (e = bx(i1, cur, plain, in_bh)) != hipSuccess) return (int)e;                 // X' = P1 X
+    if ((e = symprod(on_gram, buf_t, in_bh, in_a, SH_A - 2 * SH_B)) != hipSuccess) return (int)e;    // A2 = T P1
+    if (!all_tail && (e = syrkt(i2, cur ^ 1, plain)) != hipSuccess) return (int)e;                 // A2 = X' X'^T
+    // P2: next to T for a fused problem (P1 is still needed), over P1 otherwise
+    if ((e = syrk2(i2, every, [&](const NsProblem& P) { return P.gram_tail ? buf_p2(P) : P.Bh; })) != hipSuccess) return (int)e;
+    if ((e = symprod(on_gram, buf_p2, in_bh, buf_t, SH_B - 2 * SH_B)) != hipSuccess) return (int)e;   // Q = P2 P1 (over T)
+    // the result: Q X_{N-2} for a fused problem, P2 X_{N-1} otherwise (one launch per tile size and source buffer)
+    if ((e = bx(i2, cur, on_gram, buf_t)) != hipSuccess) return (int)e;
+    if (!all_tail && (e = bx(i2, cur ^ 1, plain, in_bh)) != hipSuccess) return (int)e;
   }
   return 0;
 }

@@ -55,7 +55,7 @@ long ns_gemm_tiles(int mode, const GemmParams& p);
 
 // tile: 256 (256x256 block tile, 8 waves) or 128 (128x128, 4 waves)
 // f16: 0 = the workspace matrices of the launch are bfloat16; 1 = IEEE half (see GemmParams::out_shift), not with split;
-// 2 = bfloat16 operands, IEEE-half result (MODE_BX with an addend, not the final launch)
+// 2 = bfloat16 operands, IEEE-half result (MODE_BX, not the final launch)
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
                                   hipStream_t stream, int f16 = 0);
 hipError_t launch_ns_gemm(int tile, int mode, bool split, bool final_, const GemmParams& p, hipStream_t stream);

@@ -25,6 +25,13 @@
 
 #include "ns_gemm.h"
 
+// The epilogue arithmetic is written out with explicit fmaf() and the compiler forms no fused operations of its own:
+// the same element is computed by different code depending on the grid (wave-local or block-cooperative epilogue,
+// 256x256 or 128x128 configuration), and all of them have to round in the same places for the result of a matrix not to
+// depend on how the launch was cut into blocks.  Left to itself the compiler fuses a multiply-add with the conversion
+// to half in one path and not in the other.
+#pragma clang fp contract(off)
+
 namespace archscale {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -45,7 +52,13 @@ __device__ __forceinline__ uint16_t bf16_bits(float f) {
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
-__device__ __forceinline__ uint16_t f16_bits(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// float -> half of a value that is ROUNDED TO FLOAT first: the empty asm keeps the compiler from merging the operation
+// that produced `f` with the conversion (v_fma_mixlo_f16 rounds the exact multiply-add result once, a separate
+// conversion rounds twice, and which of the two a code path got would otherwise depend on its shape)
+__device__ __forceinline__ uint16_t f16_bits(float f) {
+  asm("" : "+v"(f));
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
 __device__ __forceinline__ float f16_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
@@ -479,15 +492,15 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
             const float e0 = dec(e.x & 0xffff), e1 = dec(e.x >> 16);
             const float e2 = dec(e.y & 0xffff), e3 = dec(e.y >> 16);
             if (MODE == MODE_SYRK2) {
-              acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
-              acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
-              acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
-              acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
+              acc[i][j][4 * g + 0] = fmaf(alpha, acc[i][j][4 * g + 0], beta * e0);
+              acc[i][j][4 * g + 1] = fmaf(alpha, acc[i][j][4 * g + 1], beta * e1);
+              acc[i][j][4 * g + 2] = fmaf(alpha, acc[i][j][4 * g + 2], beta * e2);
+              acc[i][j][4 * g + 3] = fmaf(alpha, acc[i][j][4 * g + 3], beta * e3);
             } else {
-              acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * bx_sc;
-              acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * bx_sc;
-              acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * bx_sc;
-              acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * bx_sc;
+              acc[i][j][4 * g + 0] = fmaf(alpha, e0, acc[i][j][4 * g + 0]) * bx_sc;
+              acc[i][j][4 * g + 1] = fmaf(alpha, e1, acc[i][j][4 * g + 1]) * bx_sc;
+              acc[i][j][4 * g + 2] = fmaf(alpha, e2, acc[i][j][4 * g + 2]) * bx_sc;
+              acc[i][j][4 * g + 3] = fmaf(alpha, e3, acc[i][j][4 * g + 3]) * bx_sc;
             }
           }
         }
@@ -621,19 +634,19 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
           const float e0 = dec(e.x & 0xffff), e1 = dec(e.x >> 16);
           const float e2 = dec(e.y & 0xffff), e3 = dec(e.y >> 16);
           if (MODE == MODE_SYRK2) {
-            acc[i][j][4 * g + 0] = alpha * acc[i][j][4 * g + 0] + beta * e0;
-            acc[i][j][4 * g + 1] = alpha * acc[i][j][4 * g + 1] + beta * e1;
-            acc[i][j][4 * g + 2] = alpha * acc[i][j][4 * g + 2] + beta * e2;
-            acc[i][j][4 * g + 3] = alpha * acc[i][j][4 * g + 3] + beta * e3;
+            acc[i][j][4 * g + 0] = fmaf(alpha, acc[i][j][4 * g + 0], beta * e0);
+            acc[i][j][4 * g + 1] = fmaf(alpha, acc[i][j][4 * g + 1], beta * e1);
+            acc[i][j][4 * g + 2] = fmaf(alpha, acc[i][j][4 * g + 2], beta * e2);
+            acc[i][j][4 * g + 3] = fmaf(alpha, acc[i][j][4 * g + 3], beta * e3);
             // diagonal of the matrix (this path runs on diagonal tiles only: R0 == C0)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
               if (rl + q == cl) acc[i][j][4 * g + q] += p.diag_add;
           } else {
-            acc[i][j][4 * g + 0] = (acc[i][j][4 * g + 0] + alpha * e0) * bx_sc;
-            acc[i][j][4 * g + 1] = (acc[i][j][4 * g + 1] + alpha * e1) * bx_sc;
-            acc[i][j][4 * g + 2] = (acc[i][j][4 * g + 2] + alpha * e2) * bx_sc;
-            acc[i][j][4 * g + 3] = (acc[i][j][4 * g + 3] + alpha * e3) * bx_sc;
+            acc[i][j][4 * g + 0] = fmaf(alpha, e0, acc[i][j][4 * g + 0]) * bx_sc;
+            acc[i][j][4 * g + 1] = fmaf(alpha, e1, acc[i][j][4 * g + 1]) * bx_sc;
+            acc[i][j][4 * g + 2] = fmaf(alpha, e2, acc[i][j][4 * g + 2]) * bx_sc;
+            acc[i][j][4 * g + 3] = fmaf(alpha, e3, acc[i][j][4 * g + 3]) * bx_sc;
           }
         }
       }
@@ -745,8 +758,9 @@ template <int BM, int BN, int WM, int WN, int F16>
 static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGemmParams& p, hipStream_t s) {
   if (F16 && split) return hipErrorInvalidValue;
   if constexpr (F16 == 2) {
-    if (mode != MODE_BX || final_ || !p.g[0].E) return hipErrorInvalidValue;
-    return launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, 2>(p, s);
+    if (mode != MODE_BX || final_) return hipErrorInvalidValue;
+    return p.g[0].E ? launch_one<BM, BN, WM, WN, MODE_BX, false, false, true, 2>(p, s)
+                    : launch_one<BM, BN, WM, WN, MODE_BX, false, false, false, 2>(p, s);
   } else {
     switch (mode) {
       case MODE_SYRK:

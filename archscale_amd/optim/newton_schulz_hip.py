@@ -80,6 +80,7 @@ def newton_schulz(
     bsplit_tail: int = 0,
     normalize: bool = True,
     diag_fold: bool = True,
+    gram_tail: Optional[bool] = None,
 ) -> Tensor:
     """Orthogonalise every matrix of ``G`` (``[..., rows, cols]``, bf16 or fp32) with the quintic
     Newton-Schulz iteration ``X <- aX + (bA + cA^2)X, A = XX^T``, one ``(a, b, c)`` row per iteration.
@@ -92,6 +93,9 @@ def newton_schulz(
     last ``t`` iterations (0 = all), whose rounding dominates the error of the result.  ``normalize=False`` iterates on
     the input as it is (``epsilon`` is then unused).  ``diag_fold=False`` keeps ``aX`` as a separate addend in every
     iteration instead of storing ``B + aI`` in the iterations after the first with ``|a| <= 4.2``.
+    ``gram_tail``: with three or more iterations the last two can be stored in half and, for matrices whose long side
+    is at least twice the short one, finished on the Gram side (``X_N = P_N P_{N-1} X_{N-2}``: one ``BX`` product
+    less).  ``None`` (default) does so for ``prec="bf16"`` only, ``True`` also for "f16", ``False`` never.
     """
     _lib.require_cuda(G, "Newton-Schulz input")
     if G.dtype not in (torch.bfloat16, torch.float32):
@@ -114,6 +118,8 @@ def newton_schulz(
         flags |= _lib.NS_NO_NORMALIZE
     if not diag_fold:
         flags |= _lib.NS_NO_DIAG_FOLD
+    if gram_tail is not None:
+        flags |= _lib.NS_GRAM_TAIL if gram_tail else _lib.NS_NO_GRAM_TAIL
     with torch.cuda.device(G.device):
         st = L.muon_ns_batched(
             Gv.data_ptr(), _lib.dtype_code(Gv.dtype), bstride, ld,
@@ -135,6 +141,7 @@ def newton_schulz_grouped(
     cast_input_first: bool = True,
     outs: Optional[Sequence[Tensor]] = None,
     bsplit_tail: int = 0,
+    gram_tail: Optional[bool] = None,
 ) -> Sequence[Tensor]:
     """Orthogonalise several batches of DIFFERENT shapes in one call: every product of the iteration is a
     single kernel launch over the tiles of all batches (15 GEMM launches in total for five iterations).
@@ -165,6 +172,8 @@ def newton_schulz_grouped(
     pm = _PREC[prec]
     ws = _lib.workspace(device, L.muon_ns_grouped_workspace_bytes(probs, len(views), pm))
     flags = (_lib.NS_CAST_INPUT_FIRST if cast_input_first else 0) | _lib.ns_bsplit_tail(bsplit_tail)
+    if gram_tail is not None:
+        flags |= _lib.NS_GRAM_TAIL if gram_tail else _lib.NS_NO_GRAM_TAIL
     with torch.cuda.device(device):
         st = L.muon_ns_grouped(probs, len(views), _lib.abc_array(coeffs), len(coeffs), _as_float(epsilon),
                                _EPS[eps_mode], pm, flags, ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(device))

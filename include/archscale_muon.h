@@ -31,7 +31,8 @@ extern "C" {
 #define MUON_EPS_CLAMP 1 /* X / max(|X|, eps)    emerging_optimizers/.../spectral_ball_utils.py:46 */
 
 /* precision of B = bA + cA^2 as an operand of B*X */
-#define MUON_PREC_BF16 0       /* one bf16 rounding per GEMM epilogue (rounding points of newton_schulz_triton.py:374-378) */
+#define MUON_PREC_BF16 0       /* one bf16 rounding per GEMM epilogue (rounding points of newton_schulz_triton.py:374-378);
+                                  the last two iterations round to IEEE half instead unless MUON_NS_NO_GRAM_TAIL is set */
 #define MUON_PREC_BF16_BSPLIT 1 /* B kept as a bf16 hi+lo pair, B*X accumulates both (needed for the constant-coefficient table) */
 #define MUON_PREC_F16 2         /* the iterate and both Gram-side matrices are kept in IEEE half inside the workspace (inputs
                                    and the result stay bfloat16), each times a power of two that keeps it in the normal
@@ -50,6 +51,16 @@ extern "C" {
                                       of B; with MUON_PREC_BF16_BSPLIT only in the iterations that keep the hi+lo pair,
                                       where it is exact) and computes X' = (B + aI) X, which saves reading X a second
                                       time */
+#define MUON_NS_NO_GRAM_TAIL 8      /* keep the last two iterations as plain iterations in the storage type of prec_mode */
+#define MUON_NS_GRAM_TAIL 16        /* take the tail described below also under MUON_PREC_F16 */
+/* The tail: a call with at least three iterations whose last two rows have |a| <= 4.2 (MUON_NS_NO_DIAG_FOLD not set,
+ * input normalised, no hi+lo pair) (1) keeps the matrices of the last two iterations in IEEE half also under
+ * MUON_PREC_BF16, and (2) for every problem with long side >= 2 x short side finishes on the Gram side:
+ * X_N = (P_N P_{N-1}) X_{N-2} with A_{N-1} = P_{N-1} A_{N-2} P_{N-1}, P = aI + bA + cA^2 - three m x m symmetric
+ * products instead of one B X and one X X^T product (3 m^2 (n - m) multiply-adds less per matrix).  Default: on under
+ * MUON_PREC_BF16 (error against an fp64 run lower than with five plain bfloat16 iterations on every spectrum tried:
+ * Gaussian, rank-one spikes, log-spaced, low rank plus noise), off under MUON_PREC_F16 (there it costs 1-2 % of
+ * accuracy, 25 % with the polar-express table of msign). */
 #define MUON_NS_BSPLIT_TAIL(t) (((t) & 0xff) << 8) /* with MUON_PREC_BF16_BSPLIT: only the last t iterations keep B as a
                                                       hi+lo pair (0 = all); the rounding of B in the last iterations
                                                       dominates the error of the result */

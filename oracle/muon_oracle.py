@@ -122,6 +122,7 @@ def newton_schulz(
     *,
     eps_mode: str = "add",
     storage: str = "fp32",
+    gram_tail: Optional[bool] = None,
 ) -> Tensor:
     """Quintic Newton-Schulz  X <- aX + (bA + cA^2)X,  A = X X^T.
 
@@ -141,8 +142,14 @@ def newton_schulz(
              "bf16_gemm_bsplit": as bf16_gemm but B kept as a bf16 hi+lo pair
              "f16_gemm":    a model of the HIP path's half-precision workspace (no counterpart in the reference): one
                             IEEE-half rounding per GEMM epilogue with X, A, B kept times 2^sx, 2^8, 2^6
-                            (sx = floor(log2 sqrt(m n)) - 3), a*I inside B after the first iteration where |a| <= 4.2,
-                            bf16 result; the first iteration runs on the exact input with A and B in bf16
+                            (sx = floor(log2 sqrt(m n)) - 3), bf16 result; the first iteration runs on the exact input
+                            with A and B in bf16
+             "bf16_gemm" and "f16_gemm" also model two more choices of the HIP path (no counterpart in the
+             reference): a*I inside B in the iterations after the first with |a| <= 4.2, and, with ``gram_tail`` (None:
+             "bf16_gemm" only) and at least three iterations whose last two rows have |a| <= 4.2, the last two
+             iterations in half storage and,
+             when n >= 2m, on the Gram side: X_N = (P_N P_{N-1}) X_{N-2}, A_{N-1} = P_{N-1} A_{N-2} P_{N-1},
+             P = aI + bA + cA^2.
     Returns bf16 for the bf16 / f16 modes and fp32 for "fp32", shaped like G.
     """
     if G.ndim < 2:
@@ -168,35 +175,47 @@ def newton_schulz(
                 A = X @ X.mT
                 B = b * A + c * (A @ A)
                 X = a * X + B @ X
-        elif storage in ("bf16_gemm", "bf16_gemm_bsplit"):
+        elif storage == "bf16_gemm_bsplit":
             for a, b, c in coeffs:
                 A = _bf16_round(X @ X.mT)
                 B = c * (A @ A) + b * A
-                if storage == "bf16_gemm":
-                    X = _bf16_round(a * X + _bf16_round(B) @ X)
-                else:
-                    hi = _bf16_round(B)
-                    lo = _bf16_round(B - hi)
-                    X = _bf16_round(a * X + hi @ X + lo @ X)
+                hi = _bf16_round(B)
+                lo = _bf16_round(B - hi)
+                X = _bf16_round(a * X + hi @ X + lo @ X)
             X = X.to(torch.bfloat16)
-        elif storage == "f16_gemm":
+        elif storage in ("bf16_gemm", "f16_gemm"):
             m, n = X.shape[-2], X.shape[-1]
+            N = len(coeffs)
             sx = max(int(math.floor(0.5 * math.log2(m * n))) - 3, 0)
 
             def half(t: Tensor, shift: int) -> Tensor:
                 return (t * 2.0 ** shift).to(torch.float16).to(torch.float32) * 2.0 ** -shift
 
+            def fold_ok(it: int) -> bool:
+                return it > 0 and abs(coeffs[it][0]) <= 4.2
+
+            wanted = (storage == "bf16_gemm") if gram_tail is None else gram_tail
+            tail = wanted and N >= 3 and fold_ok(N - 2) and fold_ok(N - 1)
+            first_half = 1 if storage == "f16_gemm" else (N - 2 if tail else N)
             eye = torch.eye(m, dtype=torch.float32)
             for it, (a, b, c) in enumerate(coeffs):
-                first = it == 0
-                A = _bf16_round(X @ X.mT) if first else half(X @ X.mT, 8)
+                last = it == N - 1
+                half_ops = it >= first_half
+                half_out = not last and it + 1 >= first_half
+                rA = (lambda t: half(t, 8)) if half_ops else _bf16_round
+                rB = (lambda t: half(t, 6)) if half_ops else _bf16_round
+                A = rA(X @ X.mT)
+                if tail and n >= 2 * m and it == N - 2:
+                    a2, b2, c2 = coeffs[N - 1]
+                    P1 = rB(c * (A @ A) + b * A + a * eye)
+                    T = rB(P1 @ A)
+                    A2 = rA(T @ P1)
+                    P2 = rB(c2 * (A2 @ A2) + b2 * A2 + a2 * eye)
+                    X = _bf16_round(rB(P2 @ P1) @ X)
+                    break
                 B = c * (A @ A) + b * A
-                last = it == len(coeffs) - 1
-                if it > 0 and abs(a) <= 4.2:
-                    Y = half(B + a * eye, 6) @ X
-                else:
-                    Y = a * X + (_bf16_round(B) if first else half(B, 6)) @ X
-                X = _bf16_round(Y) if last else half(Y, sx)
+                Y = rB(B + a * eye) @ X if fold_ok(it) else a * X + rB(B) @ X
+                X = half(Y, sx) if half_out else _bf16_round(Y)
             X = X.to(torch.bfloat16)
         else:
             raise ValueError(f"unknown storage {storage!r}")

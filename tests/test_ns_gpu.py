@@ -372,7 +372,7 @@ def test_half_precision_workspace(ns, gpu_device, shape, table):
     coeffs = O.coefficient_schedule(table, 5)
     em = "clamp" if table == "msign" else "add"
     got = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, eps_mode=em, prec="f16")
-    plain = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, eps_mode=em, prec="bf16")
+    plain = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, eps_mode=em, prec="bf16", gram_tail=False)   # bf16 storage throughout
     torch.cuda.synchronize()
     assert got.dtype == torch.bfloat16 and got.shape == G.shape
     mats = G if G.ndim == 3 else G[None]
@@ -430,3 +430,53 @@ def test_emerging_newton_schulz_named_sets(gpu_device, kind, steps, shape):
     # an explicit transpose flag (either value) changes nothing
     flipped = newton_schulz(x.to(gpu_device), steps, kind, custom, transpose=shape[-2] <= shape[-1])
     assert torch.equal(flipped, got)
+
+
+@pytest.mark.parametrize("shape", [(512, 2048), (2048, 256), (320, 1100), (3, 136, 400), (256, 512), (300, 599)])
+@pytest.mark.parametrize("prec,table", [("bf16", "quintic"), ("f16", "quintic"), ("f16", "simple")])
+def test_gram_side_tail(ns, gpu_device, shape, prec, table):
+    """The last two iterations in half storage and, for n >= 2m, on the Gram side (the default) against the same call
+    with plain last iterations and against the fp32 oracle: no further from the oracle than the plain path."""
+    print("case", shape, prec, table, flush=True)
+    G = _randn(shape, 31 + sum(shape))
+    coeffs = O.coefficient_schedule(table, 5)
+    want = O.newton_schulz(G, coeffs, 1e-7, storage="fp32")
+    got = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, prec=prec, gram_tail=True)
+    plain = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, prec=prec, gram_tail=False)
+    auto = ns.newton_schulz(G.to(gpu_device), coeffs, 1e-7, prec=prec)
+    torch.cuda.synchronize()
+    assert torch.equal(auto, got if prec == "bf16" else plain)      # the default: on for bf16 storage, off for half
+    e1, e0 = _rel(got, want), _rel(plain, want)
+    print("rel err with / without the tail", e1, e0, flush=True)
+    assert e1 <= NS_TOL and e1 <= 1.1 * e0 + 2e-4
+    m, n = min(shape[-2:]), max(shape[-2:])
+    if n >= 2 * m or prec == "bf16":
+        assert not torch.equal(got, plain)       # the default really took the other path
+    else:
+        assert torch.equal(got, plain)           # half workspace, n < 2m: nothing changes
+    model = O.newton_schulz(G, coeffs, 1e-7, storage="f16_gemm" if prec == "f16" else "bf16_gemm", gram_tail=True)
+    assert _rel(got, model.float()) <= (2.5e-3 if prec == "f16" else 6e-3)
+
+
+def test_gram_side_tail_spiked_and_grouped(ns, gpu_device):
+    """A gradient with a dominant direction (Gaussian plus a 30x rank-one spike), and a grouped call that mixes classes
+    that take the Gram-side tail with classes that do not: every problem equals its own single call bit for bit."""
+    g = torch.Generator().manual_seed(5)
+    spike = (torch.randn(512, 2048, generator=g) + 30 * torch.randn(512, 1, generator=g) @ torch.randn(1, 2048, generator=g))
+    spike = spike.to(torch.bfloat16)
+    want = O.newton_schulz(spike, O.QUINTIC, 1e-7, storage="fp32")
+    for prec, bar in (("bf16", 8e-3), ("f16", 3e-3)):
+        got = ns.newton_schulz(spike.to(gpu_device), O.QUINTIC, 1e-7, prec=prec, gram_tail=True)
+        plain = ns.newton_schulz(spike.to(gpu_device), O.QUINTIC, 1e-7, prec=prec, gram_tail=False)
+        e1, e0 = _rel(got, want), _rel(plain, want)
+        print("spike", prec, e1, e0, flush=True)
+        assert e1 <= bar and e1 <= 1.1 * e0 + 2e-4
+    shapes = [(2, 256, 1024), (384, 384), (640, 256), (3, 300, 700), (512, 600)]
+    ins = [_randn(s, 100 + i).to(gpu_device) for i, s in enumerate(shapes)]
+    for prec in ("bf16", "f16"):
+        outs = ns.newton_schulz_grouped(ins, O.QUINTIC, 1e-7, prec=prec, gram_tail=True)
+        torch.cuda.synchronize()
+        for x, o in zip(ins, outs):
+            single = ns.newton_schulz(x, O.QUINTIC, 1e-7, prec=prec, gram_tail=True)
+            assert torch.equal(o, single), (prec, tuple(x.shape))
+            assert _rel(o, O.newton_schulz(x.cpu(), O.QUINTIC, 1e-7, storage="fp32")) <= NS_TOL

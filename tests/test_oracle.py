@@ -148,6 +148,47 @@ def test_ns_bf16_modes_close_to_fp32(table, storage, bar):
     assert got.dtype == torch.float32 and (got - ref).norm() / ref.norm() < bar
 
 
+def test_gram_tail_is_the_same_map():
+    """The last two iterations on the Gram side, X_N = (P_N P_{N-1}) X_{N-2} with A_{N-1} = P_{N-1} A_{N-2} P_{N-1} and
+    P = aI + bA + cA^2, against two plain iterations in fp64 (a transposed factor, a wrong power of P or the wrong
+    coefficient row in P_N fails this), and the storage models with and without it against the fp32 run."""
+    g = torch.Generator().manual_seed(21)
+    X = torch.randn(12, 40, generator=g, dtype=torch.float64)
+    X = X / X.norm()
+    (a1, b1, c1), (a2, b2, c2) = O.QUINTIC[3], O.QUINTIC[4]
+    plain = X
+    for a, b, c in ((a1, b1, c1), (a2, b2, c2)):
+        A = plain @ plain.mT
+        plain = a * plain + (b * A + c * (A @ A)) @ plain
+    eye = torch.eye(12, dtype=torch.float64)
+    A = X @ X.mT
+    P1 = a1 * eye + b1 * A + c1 * (A @ A)
+    A2 = (P1 @ A) @ P1
+    P2 = a2 * eye + b2 * A2 + c2 * (A2 @ A2)
+    assert torch.allclose((P2 @ P1) @ X, plain, rtol=1e-12, atol=1e-14)
+    G = torch.randn(96, 320, generator=g)          # n >= 2m: the models take the Gram-side tail
+    for table, storage, bar in (("quintic", "bf16_gemm", 6e-3), ("simple", "f16_gemm", 4e-3), ("quintic", "f16_gemm", 4e-3)):
+        c = O.coefficient_schedule(table, 5)
+        ref = O.newton_schulz(G, c, 1e-7, storage="fp32")
+        with_tail = O.newton_schulz(G, c, 1e-7, storage=storage, gram_tail=True).float()
+        without = O.newton_schulz(G, c, 1e-7, storage=storage, gram_tail=False).float()
+        e1 = ((with_tail - ref).norm() / ref.norm()).item()
+        e0 = ((without - ref).norm() / ref.norm()).item()
+        assert e1 < bar and e1 < 1.15 * e0 + 2e-4, (table, storage, e1, e0)
+        assert not torch.equal(with_tail, without)
+    # a large `a` in the last rows (no a*I inside B there) or fewer than three iterations: no tail
+    big = [(3.0, -3.2, 1.2), (2.0, -1.5, 0.5), (5.0, -3.0, 0.5)]
+    assert torch.equal(O.newton_schulz(G, big, 1e-7, storage="bf16_gemm"),
+                       O.newton_schulz(G, big, 1e-7, storage="bf16_gemm", gram_tail=False))
+    two = O.coefficient_schedule("quintic", 2)
+    assert torch.equal(O.newton_schulz(G, two, 1e-7, storage="f16_gemm", gram_tail=True),
+                       O.newton_schulz(G, two, 1e-7, storage="f16_gemm", gram_tail=False))
+    # default: the bfloat16 model takes it, the half model does not
+    c = O.coefficient_schedule("quintic", 5)
+    assert torch.equal(O.newton_schulz(G, c, 1e-7, storage="bf16_gemm"), O.newton_schulz(G, c, 1e-7, storage="bf16_gemm", gram_tail=True))
+    assert torch.equal(O.newton_schulz(G, c, 1e-7, storage="f16_gemm"), O.newton_schulz(G, c, 1e-7, storage="f16_gemm", gram_tail=False))
+
+
 def test_msign_contract():
     G = torch.randn(16, 48)
     with pytest.raises(ValueError):
