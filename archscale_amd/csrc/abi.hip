@@ -378,7 +378,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const muon_mns_problem& f = fused[i];
     const long xs = (long)pl.Mp * pl.Np;
     const int d_rows = P.tall ? pl.Np : pl.Mp, d_cols = P.tall ? pl.Mp : pl.Np;   // padded extents of the matrix itself
-    const int tiles = (d_rows / MOMLAY_TILE) * (d_cols / MOMLAY_TILE);
+    // a tall matrix whose extents need no padding goes into the workspace as it is: a linear pass, partials per chunk
+    const bool linear = P.tall && P.q.rows == pl.Np && P.q.cols == pl.Mp;
+    const int tiles = linear ? pl.cpm : (d_rows / MOMLAY_TILE) * (d_cols / MOMLAY_TILE);
     for (int b0 = 0; b0 < P.q.batch; b0 += MOMLAY_MAX) {
       MomLayoutParams mp = {};
       mp.n_mats = std::min(MOMLAY_MAX, P.q.batch - b0);
@@ -397,7 +399,8 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       // algorithmic bytes: G read, M read and written, the operand image written (2 bytes each)
       const double esz = (double)mp.n_mats * P.q.rows * P.q.cols;
       const double bytes = esz * ((f.g_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2 * (f.m_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2);
-      e = timed_launch(PROF_KEY_MOMENTUM_LAYOUT, bytes, bytes, stream, [&] { return launch_momentum_layout(mp, stream); });
+      e = timed_launch(PROF_KEY_MOMENTUM_LAYOUT, bytes, bytes, stream,
+                       [&] { return linear ? launch_momentum_linear(mp, stream) : launch_momentum_layout(mp, stream); });
       if (e != hipSuccess) return (int)e;
     }
     e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);

@@ -63,6 +63,9 @@ struct MomLayoutParams {
   const void* w[MOMLAY_MAX];     // read only when c.l2 != 0
 };
 hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream);
+// the case without transposition and padding (dst[mat] laid out like the source): linear chunks of MUON_CHUNK_ELEMS,
+// p.partial = [n_mats][ceil(rows * cols / MUON_CHUNK_ELEMS)]
+hipError_t launch_momentum_linear(const MomLayoutParams& p, hipStream_t stream);
 hipError_t launch_norm_scale_from_partials(const float* partial, int partials_per_mat, int batch, float eps, int eps_mode,
                                            float* scale, hipStream_t stream);
 

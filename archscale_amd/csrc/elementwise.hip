@@ -109,8 +109,10 @@ __device__ __forceinline__ void block_reduce(float (&v)[N], float* smem /* N * 4
 //    lit_gpt: (mu, 1, mu|1, 1|0)  (muon.py:665-679);  emerging: (b, 1-b, b|1, 1-b|0)
 //    (orthogonalized_optimizer.py:193-199, mixin.py:48-49 for the l2 term)
 // ---------------------------------------------------------------------------
-template <int GD, int MD, int UD>
-__device__ __forceinline__ void momentum_range(const PreItem& it, long begin, long end, const MomentumCoef c, bool vec_ok) {
+// SS: also accumulate the sum of squares of the update as stored (rounded to U's dtype) into `ss`
+template <int GD, int MD, int UD, bool SS = false>
+__device__ __forceinline__ void momentum_range(const PreItem& it, long begin, long end, const MomentumCoef c, bool vec_ok,
+                                               float* ss = nullptr) {
   const void* g = it.g; void* m = it.m; void* u = it.u;
   if (vec_ok) {
 #pragma unroll
@@ -133,6 +135,7 @@ __device__ __forceinline__ void momentum_range(const PreItem& it, long begin, lo
           const float mn = Elem<MD>::round(fmaf(c.mm, mv[k], c.mg * gm));
           mv[k] = mn;
           uv[k] = fmaf(c.um, mn, c.ug * gm);
+          if (SS) { const float x = Elem<UD>::round(uv[k]); *ss += x * x; }
         }
         Elem<MD>::store8(m, i, mv);
         Elem<UD>::store8(u, i, uv);
@@ -149,7 +152,9 @@ __device__ __forceinline__ void momentum_range(const PreItem& it, long begin, lo
       const float gm = Elem<MD>::round(gv);
       const float mn = Elem<MD>::round(fmaf(c.mm, Elem<MD>::load1(m, i), c.mg * gm));
       Elem<MD>::store1(m, i, mn);
-      Elem<UD>::store1(u, i, fmaf(c.um, mn, c.ug * gm));
+      const float uv = fmaf(c.um, mn, c.ug * gm);
+      Elem<UD>::store1(u, i, uv);
+      if (SS) { const float x = Elem<UD>::round(uv); *ss += x * x; }
     }
   }
 }
@@ -489,6 +494,43 @@ hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream) 
     return hipErrorInvalidValue;
   hipLaunchKernelGGL(momentum_layout_kernel, dim3(p.d_cols / MOMLAY_TILE, p.d_rows / MOMLAY_TILE, p.n_mats), dim3(256), 0,
                      stream, p);
+  return hipGetLastError();
+}
+
+// The same when the operand image is the matrix itself (no transposition, no padding: dst[mat] has the layout of the
+// source): a linear pass in chunks of MUON_CHUNK_ELEMS like momentum_kernel, one partial sum of squares per chunk.
+// p.d_rows / p.d_cols / p.ldd are not used; p.partial holds [n_mats][chunks_per_mat] values.
+__global__ void __launch_bounds__(EW_THREADS)
+momentum_linear_kernel(const MomLayoutParams p, int chunks_per_mat) {
+  __shared__ float red[4];
+  const int mat = blockIdx.y, chunk = blockIdx.x;
+  PreItem it;
+  it.g = p.g[mat]; it.m = p.m[mat]; it.w = p.w[mat];
+  it.u = p.dst + (size_t)mat * p.d_bstride;
+  it.numel = (long)p.rows * p.cols;
+  it.g_dtype = p.g_dtype; it.m_dtype = p.m_dtype; it.u_dtype = DT_BF16; it.w_dtype = p.w_dtype;
+  const long begin = (long)chunk * MUON_CHUNK_ELEMS;
+  const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
+  const bool vec_ok = aligned16(it.g) && aligned16(it.m) && aligned16(it.u) && (p.c.l2 == 0.f || aligned16(it.w)) &&
+                      (it.numel % EW_VEC == 0);
+  float s[1] = {0.f};
+  switch ((p.g_dtype << 1) | p.m_dtype) {
+    case 0: momentum_range<DT_BF16, DT_BF16, DT_BF16, true>(it, begin, end, p.c, vec_ok, &s[0]); break;
+    case 1: momentum_range<DT_BF16, DT_F32, DT_BF16, true>(it, begin, end, p.c, vec_ok, &s[0]); break;
+    case 2: momentum_range<DT_F32, DT_BF16, DT_BF16, true>(it, begin, end, p.c, vec_ok, &s[0]); break;
+    default: momentum_range<DT_F32, DT_F32, DT_BF16, true>(it, begin, end, p.c, vec_ok, &s[0]); break;
+  }
+  block_reduce<1>(s, red);
+  if (threadIdx.x == 0) p.partial[(size_t)mat * chunks_per_mat + chunk] = s[0];
+}
+
+hipError_t launch_momentum_linear(const MomLayoutParams& p, hipStream_t stream) {
+  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.rows < 1 || p.cols < 1 || p.transpose) return hipErrorInvalidValue;
+  const long numel = (long)p.rows * p.cols;
+  if (p.d_bstride < numel) return hipErrorInvalidValue;
+  const long cpm = (numel + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS;
+  if (cpm > 0x7fffffffL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(momentum_linear_kernel, dim3((unsigned)cpm, p.n_mats), dim3(EW_THREADS), 0, stream, p, (int)cpm);
   return hipGetLastError();
 }
 

@@ -398,6 +398,14 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const float bx_sc = sc * __builtin_ldexpf(1.f, p.out_shift);   // MODE_BX: scale of the result (a power of two from the host)
   const float alpha = SYRK_PLAIN ? p.alpha * sc * sc : p.alpha, beta = p.beta;
   const bool diag = SYM && (ti == tj);
+  // A diagonal tile of a product of a matrix with ITSELF is symmetric bit for bit as it comes out of the matrix cores
+  // (element (i,j) and element (j,i) are the same products summed in the same order over k), so it takes the wave-local
+  // epilogue below like any other tile and writes one image.  A diagonal tile of P Q^T with two different (commuting,
+  // symmetric) matrices is symmetric only up to rounding: it keeps its upper half and reflects it.
+  const bool self_product = p.P == p.Q && p.strideP == p.strideQ && p.ldp == p.ldq;
+  // (the instantiation that writes a hi+lo pair keeps the reflecting path for every diagonal tile: its epilogue has no
+  // registers to spare for the diagonal term in the wave-local one)
+  const bool reflect = diag && (!self_product || (SPLIT && MODE == MODE_SYRK2));
   // S[cl][rl]: chunk index XOR cl, so the 32 lanes of an 8-byte access (32 different cl) spread over all banks
   auto s_off = [](int cl, int rl) { return cl * TPITCH + ((((rl >> 3) ^ cl) & (CPRT - 1)) << 4) + ((rl & 7) << 1); };
   auto s_chunk = [](int cl, int ch) { return cl * TPITCH + (((ch ^ cl) & (CPRT - 1)) << 4); };
@@ -434,8 +442,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 
   __syncthreads();  // every wave is done reading the operand stages
 
-  if (!diag) {
-    // ---- wave-local epilogue (every tile except the diagonal tiles of a symmetric product).
+  if (!reflect) {
+    // ---- wave-local epilogue (every tile except the diagonal tiles of a product of two different matrices).
     // Each wave stages its own WM x WN sub-tile in its own LDS region as the transposed image
     // W[c][r] (c = column in the sub-tile, r = row), so nothing below needs a block barrier:
     //   addend in:   16-byte direct copies of E[col][row..] rows into W, read back 8 bytes per lane
@@ -506,6 +514,27 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
         }
       }
 
+    if constexpr (MODE == MODE_SYRK2 && !SPLIT) {
+      // B + a I: in a diagonal tile (R0 == C0) the diagonal of the matrix runs through the 32x32 blocks (j + d32, j) of
+      // this wave's sub-tile with 32 d32 == wc0 - wr0, where it is the element with 8*g + q == l32 - 4*hi.  Only those
+      // blocks are touched, with a select per element.
+      const int d32 = (wc0 - wr0) / 32;   // wave-uniform
+      if (diag && d32 >= 0 && (wc0 - wr0) % 32 == 0) {
+        const int t = l32 - 4 * hi;
+        const float da = p.diag_add;
+#pragma unroll
+        for (int dd = 0; dd < FM; ++dd)
+          if (dd == d32) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+              if (j + dd < FM) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[j + dd][j][e] += (8 * (e >> 2) + (e & 3) == t) ? da : 0.f;
+              }
+          }
+      }
+    }
+
     auto store_wave = [&](__bf16* Cdst, int lane) {
       const int l32 = lane & 31, hi = lane >> 5;
       // W[c][r] <- bf16(acc)
@@ -519,7 +548,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
                 pk4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
       // transposed / mirrored image: rows of W
       __bf16* Tdst = SYM ? Cdst : p.Ct;
-      if (Tdst) {
+      if (Tdst && !diag) {   // a diagonal tile is its own mirror image
         const long tbs = SYM ? p.strideC : p.strideCt;
         const int tld = SYM ? p.ldc : p.ldct;
         __bf16* base = Tdst + (size_t)b * tbs;
