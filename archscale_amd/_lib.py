@@ -5,6 +5,7 @@ There is no fallback: if the library is missing or a call fails, this raises.
 from __future__ import annotations
 
 import ctypes
+import math
 import os
 import threading
 from typing import Dict, Optional, Sequence, Tuple
@@ -44,6 +45,10 @@ SCALAR_ITEM = np.dtype(
 BALL_ITEM = np.dtype(
     [("w", "<u8"), ("phi", "<u8"), ("sigma", "<u8"), ("ld_w", "<i8"), ("ld_phi", "<i8"), ("rows", "<i4"), ("cols", "<i4"),
      ("radius", "<f4"), ("lr_ratio", "<f4"), ("w_dtype", "<i4"), ("reserved", "<i4")], align=True)
+#: muon_hyper: the hyper-parameter block the *_dev entry points read from device memory
+HYPER = np.dtype([("lr", "<f4"), ("lr_wd", "<f4"), ("eps", "<f4"), ("w1", "<f4"), ("w2", "<f4"), ("bias1", "<f4"),
+                  ("bias2_sqrt", "<f4"), ("cautious", "<i4")], align=True)
+assert HYPER.itemsize == 32
 assert PRE_ITEM.itemsize == 56 and POST_ITEM.itemsize == 32 and SCALAR_ITEM.itemsize == 56 and BALL_ITEM.itemsize == 64
 
 
@@ -132,6 +137,13 @@ _SIGNATURES = {
     "muon_update_muonh": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
         ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+    "muon_update_plain_dev": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
+    "muon_update_muonh_dev": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+    "muon_scalar_update_dev": (ctypes.c_int, [
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+        ctypes.c_void_p, ctypes.c_void_p]),
     "muon_spectral_norm_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(SnProblem), ctypes.c_int]),
     "muon_spectral_norm": (ctypes.c_int, [
         ctypes.POINTER(SnProblem), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
@@ -179,6 +191,21 @@ def check(status: int, what: str) -> None:
         if status < 0:
             raise ValueError(f"{what}: {msg}")
         raise MuonLibraryError(f"{what}: HIP error {status}: {msg}")
+
+
+def hyper_record(lr: float, lr_wd: float, eps: float = 0.0, beta1: float = 0.0, beta2: float = 0.0, step: int = 1,
+                 cautious: bool = False) -> np.ndarray:
+    """One muon_hyper record with the derived fields computed exactly as the by-value entry points compute them
+    (w1, w2 in float arithmetic on the float-rounded betas; the bias corrections in double, then rounded)."""
+    rec = np.zeros(1, dtype=HYPER)
+    b1, b2 = np.float32(beta1), np.float32(beta2)
+    rec["lr"], rec["lr_wd"], rec["eps"] = lr, lr_wd, eps
+    rec["w1"], rec["w2"] = np.float32(1.0) - b1, np.float32(1.0) - b2
+    step = max(int(step), 1)
+    rec["bias1"] = 1.0 - float(b1) ** step
+    rec["bias2_sqrt"] = math.sqrt(1.0 - float(b2) ** step)
+    rec["cautious"] = int(bool(cautious))
+    return rec
 
 
 def ns_bsplit_tail(t: int) -> int:

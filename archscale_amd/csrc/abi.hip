@@ -559,11 +559,13 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       return true;
     });
   };
-  // X' = a X + B X with B = lhs(P) and X^T in Xt[src]; the next iterate goes to Xt[src ^ 1], the last one to the caller
-  auto bx = [&](int it, int src, auto&& want, auto&& lhs) -> hipError_t {
+  // X' = a X + B X with B = lhs(P) and X^T in Xt[src_of(P)]; the next iterate goes to the other X^T buffer, the last
+  // one to the caller
+  auto bx = [&](int it, auto&& src_of, auto&& want, auto&& lhs) -> hipError_t {
     const ItCfg k = it_cfg(it);
     return run_mode(MODE_BX, k.split, k.last, k.bx16, [&](const NsProblem& P, GemmParams& g, double& fa, double& fi) {
       if (!want(P)) return false;
+      const int src = src_of(P);
       const NsPlan& pl = P.pl;
       const long xs = (long)pl.Mp * pl.Np, as = (long)pl.Mp * pl.Mp;
       g.batch = P.q.batch;
@@ -598,7 +600,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   for (int it = 0; it < n_plain_iters; ++it) {
     if ((e = syrkt(it, cur, every)) != hipSuccess) return (int)e;
     if ((e = syrk2(it, every, in_bh)) != hipSuccess) return (int)e;
-    if ((e = bx(it, cur, every, in_bh)) != hipSuccess) return (int)e;
+    if ((e = bx(it, [&](const NsProblem&) { return cur; }, every, in_bh)) != hipSuccess) return (int)e;
     cur ^= 1;
   }
   if (any_tail) {
@@ -610,15 +612,16 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     if ((e = syrkt(i1, cur, every)) != hipSuccess) return (int)e;                                  // A1 = X X^T
     if ((e = syrk2(i1, every, in_bh)) != hipSuccess) return (int)e;                                // P1 (in Bh)
     if ((e = symprod(on_gram, in_bh, in_a, buf_t, SH_B - SH_B - SH_A)) != hipSuccess) return (int)e;  // T = P1 A1
-    if (!all_tail && (e = bx(i1, cur, plain, in_bh)) != hipSuccess) return (int)e;                 // X' = P1 X
+    if (!all_tail && (e = bx(i1, [&](const NsProblem&) { return cur; }, plain, in_bh)) != hipSuccess) return (int)e;  // X' = P1 X
     if ((e = symprod(on_gram, buf_t, in_bh, in_a, SH_A - 2 * SH_B)) != hipSuccess) return (int)e;    // A2 = T P1
     if (!all_tail && (e = syrkt(i2, cur ^ 1, plain)) != hipSuccess) return (int)e;                 // A2 = X' X'^T
     // P2: next to T for a fused problem (P1 is still needed), over P1 otherwise
     if ((e = syrk2(i2, every, [&](const NsProblem& P) { return P.gram_tail ? buf_p2(P) : P.Bh; })) != hipSuccess) return (int)e;
     if ((e = symprod(on_gram, buf_p2, in_bh, buf_t, SH_B - 2 * SH_B)) != hipSuccess) return (int)e;   // Q = P2 P1 (over T)
-    // the result: Q X_{N-2} for a fused problem, P2 X_{N-1} otherwise (one launch per tile size and source buffer)
-    if ((e = bx(i2, cur, on_gram, buf_t)) != hipSuccess) return (int)e;
-    if (!all_tail && (e = bx(i2, cur ^ 1, plain, in_bh)) != hipSuccess) return (int)e;
+    // the result, one launch for all: Q X_{N-2} for a fused problem, P2 X_{N-1} otherwise
+    e = bx(i2, [&](const NsProblem& P) { return P.gram_tail ? cur : cur ^ 1; }, every,
+           [&](const NsProblem& P) { return P.gram_tail ? buf_t(P) : P.Bh; });
+    if (e != hipSuccess) return (int)e;
   }
   return 0;
 }
@@ -738,6 +741,17 @@ int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_
   h.cautious = cautious;
   return (int)launch_scalar_update(items_dev, prefix_dev, n_items, total_chunks, algo, hyperball, h, scratch_dev,
                                    (hipStream_t)stream);
+}
+
+int muon_scalar_update_dev(const muon_scalar_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                           int algo, int hyperball, const muon_hyper* hyper_dev, float* scratch_dev, void* stream) {
+  if (n_items == 0) return 0;
+  if (!items_dev || !prefix_dev || !hyper_dev || n_items < 0 || total_chunks < n_items) return MUON_E_ARG;
+  if (((uintptr_t)hyper_dev & 3) != 0) return MUON_E_ARG;
+  if (algo != MUON_ALGO_ADAMW && algo != MUON_ALGO_LION) return MUON_E_ARG;
+  if (hyperball && (algo != MUON_ALGO_ADAMW || !scratch_dev || ((uintptr_t)scratch_dev & 7))) return MUON_E_ARG;
+  return (int)launch_scalar_update(items_dev, prefix_dev, n_items, total_chunks, algo, hyperball, ScalarHyper{}, scratch_dev,
+                                   (hipStream_t)stream, hyper_dev);
 }
 
 // ---- MuonBall -------------------------------------------------------------------------------------------
@@ -979,6 +993,24 @@ int muon_update_plain(const muon_post_item* items_dev, const int32_t* prefix_dev
   if (!items_dev || !prefix_dev || n_items < 0 || total_chunks < n_items) return MUON_E_ARG;
   return (int)launch_post_plain(items_dev, prefix_dev, n_items, total_chunks, lr, lr_wd, cautious,
                                 (hipStream_t)stream);
+}
+
+int muon_update_plain_dev(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                          const muon_hyper* hyper_dev, void* stream) {
+  if (n_items == 0) return 0;
+  if (!items_dev || !prefix_dev || !hyper_dev || n_items < 0 || total_chunks < n_items) return MUON_E_ARG;
+  if (((uintptr_t)hyper_dev & 3) != 0) return MUON_E_ARG;
+  return (int)launch_post_plain(items_dev, prefix_dev, n_items, total_chunks, 0.f, 0.f, 0, (hipStream_t)stream, hyper_dev);
+}
+
+int muon_update_muonh_dev(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                          const muon_hyper* hyper_dev, float* scratch_dev, void* stream) {
+  if (n_items == 0) return 0;
+  if (!items_dev || !prefix_dev || !hyper_dev || !scratch_dev || n_items < 0 || total_chunks < n_items) return MUON_E_ARG;
+  if (((uintptr_t)hyper_dev & 3) != 0) return MUON_E_ARG;
+  if ((uintptr_t)scratch_dev & 7) return MUON_E_WORKSPACE;
+  return (int)launch_post_muonh(items_dev, prefix_dev, n_items, total_chunks, 0.f, 0.f, 0.f, 0, scratch_dev,
+                                (hipStream_t)stream, hyper_dev);
 }
 
 size_t muon_muonh_scratch_floats(int n_items, int total_chunks) {

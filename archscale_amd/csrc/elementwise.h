@@ -17,12 +17,8 @@ typedef muon_scalar_item ScalarItem;
 enum { ALGO_ADAMW = MUON_ALGO_ADAMW, ALGO_LION = MUON_ALGO_LION };
 
 // hyper-parameters of the scalar updates, precomputed on the host
-struct ScalarHyper {
-  float lr, lr_wd, eps;
-  float w1, w2;            // 1 - beta1, 1 - beta2
-  float bias1, bias2_sqrt; // 1 - beta1^step, sqrt(1 - beta2^step)
-  int cautious;
-};
+// (the layout of muon_hyper in the C ABI: the *_dev entry points hand the kernels a device pointer to one)
+typedef muon_hyper ScalarHyper;
 
 struct MomentumCoef {
   float mm, mg, um, ug, l2;
@@ -72,14 +68,18 @@ hipError_t launch_norm_scale_from_partials(const float* partial, int partials_pe
 hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
                              int batch, int rows, int cols, hipStream_t stream);
 
+// hdev (nullable, device memory): when given, the kernels take the hyper-parameters from it instead of the by-value
+// arguments, so a captured launch follows a schedule
 hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                             float lr, float lrwd, int cautious, hipStream_t stream);
+                             float lr, float lrwd, int cautious, hipStream_t stream, const ScalarHyper* hdev = nullptr);
 
 hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream);
+                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream,
+                             const ScalarHyper* hdev = nullptr);
 
 hipError_t launch_scalar_update(const ScalarItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream);
+                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream,
+                                const ScalarHyper* hdev = nullptr);
 
 hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 

@@ -605,8 +605,10 @@ __device__ __forceinline__ void post_reduce_range(const PostItem& it, long begin
 
 __global__ void __launch_bounds__(EW_THREADS)
 post_reduce_kernel(const PostItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
-                   float lrwd, int cautious, float* __restrict__ partial /* [total_chunks][3] */) {
+                   float lrwd, int cautious, float* __restrict__ partial /* [total_chunks][3] */,
+                   const ScalarHyper* __restrict__ hdev) {
   __shared__ float red[12];
+  if (hdev) { lrwd = hdev->lr_wd; cautious = hdev->cautious; }   // hyper-parameters from device memory
   const int chunk = blockIdx.x;
   const int ii = find_item(prefix, n_items, chunk);
   const PostItem it = items[ii];
@@ -627,8 +629,9 @@ post_reduce_kernel(const PostItem* __restrict__ items, const int32_t* __restrict
 // one block per item: (alpha, beta) with X <- alpha*x' + beta*U
 __global__ void __launch_bounds__(EW_THREADS)
 muonh_coef_kernel(const int32_t* __restrict__ prefix, const float* __restrict__ partial, float lr, float eps,
-                  float2* __restrict__ coef) {
+                  float2* __restrict__ coef, const ScalarHyper* __restrict__ hdev) {
   __shared__ double red[3][4];
+  if (hdev) { lr = hdev->lr; eps = hdev->eps; }
   const int ii = blockIdx.x;
   double s[3] = {0.0, 0.0, 0.0};
   for (int c = prefix[ii] + threadIdx.x; c < prefix[ii + 1]; c += EW_THREADS) {
@@ -683,7 +686,9 @@ __device__ __forceinline__ void post_apply_range(const PostItem& it, long begin,
 
 __global__ void __launch_bounds__(EW_THREADS)
 post_apply_kernel(const PostItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
-                  float lr, float lrwd, int cautious, const float2* __restrict__ coef) {
+                  float lr, float lrwd, int cautious, const float2* __restrict__ coef,
+                  const ScalarHyper* __restrict__ hdev) {
+  if (hdev) { lr = hdev->lr; lrwd = hdev->lr_wd; cautious = hdev->cautious; }
   const int chunk = blockIdx.x;
   const int ii = find_item(prefix, n_items, chunk);
   const PostItem it = items[ii];
@@ -697,23 +702,24 @@ post_apply_kernel(const PostItem* __restrict__ items, const int32_t* __restrict_
 }
 
 hipError_t launch_post_plain(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                             float lr, float lrwd, int cautious, hipStream_t stream) {
+                             float lr, float lrwd, int cautious, hipStream_t stream, const ScalarHyper* hdev) {
   if (total_chunks <= 0) return hipSuccess;
   hipLaunchKernelGGL(post_apply_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
-                     lr, lrwd, cautious, (const float2*)nullptr);
+                     lr, lrwd, cautious, (const float2*)nullptr, hdev);
   return hipGetLastError();
 }
 
 hipError_t launch_post_muonh(const PostItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream) {
+                             float lr, float lrwd, float eps, int cautious, float* scratch, hipStream_t stream,
+                             const ScalarHyper* hdev) {
   if (total_chunks <= 0) return hipSuccess;
   float* partial = scratch;                                             // 3 * total_chunks
   float2* coef = (float2*)(scratch + (size_t)3 * total_chunks + ((total_chunks & 1) ? 1 : 0));  // 8-byte aligned
   hipLaunchKernelGGL(post_reduce_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
-                     lrwd, cautious, partial);
-  hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), dim3(EW_THREADS), 0, stream, prefix, partial, lr, eps, coef);
+                     lrwd, cautious, partial, hdev);
+  hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), dim3(EW_THREADS), 0, stream, prefix, partial, lr, eps, coef, hdev);
   hipLaunchKernelGGL(post_apply_kernel, dim3(total_chunks), dim3(EW_THREADS), 0, stream, items, prefix, n_items,
-                     lr, lrwd, cautious, (const float2*)coef);
+                     lr, lrwd, cautious, (const float2*)coef, hdev);
   return hipGetLastError();
 }
 
@@ -770,8 +776,10 @@ __device__ __forceinline__ float scalar_elem(float x, float g, float& m, float& 
 template <int ALGO, int PHASE>
 __global__ void __launch_bounds__(EW_THREADS)
 scalar_update_kernel(const ScalarItem* __restrict__ items, const int32_t* __restrict__ prefix, int n_items,
-                     ScalarHyper h, float* __restrict__ partial, const float2* __restrict__ coef) {
+                     ScalarHyper h, float* __restrict__ partial, const float2* __restrict__ coef,
+                     const ScalarHyper* __restrict__ hdev) {
   __shared__ float red[12];
+  if (hdev) h = *hdev;   // hyper-parameters from device memory
   const int chunk = blockIdx.x;
   const int ii = find_item(prefix, n_items, chunk);
   const ScalarItem it = items[ii];
@@ -830,23 +838,24 @@ scalar_update_kernel(const ScalarItem* __restrict__ items, const int32_t* __rest
 }
 
 hipError_t launch_scalar_update(const ScalarItem* items, const int32_t* prefix, int n_items, int total_chunks,
-                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream) {
+                                int algo, int hyperball, ScalarHyper h, float* scratch, hipStream_t stream,
+                                const ScalarHyper* hdev) {
   if (total_chunks <= 0) return hipSuccess;
   dim3 grid(total_chunks), block(EW_THREADS);
   if (algo == ALGO_LION) {
     hipLaunchKernelGGL((scalar_update_kernel<ALGO_LION, 0>), grid, block, 0, stream, items, prefix, n_items, h,
-                       (float*)nullptr, (const float2*)nullptr);
+                       (float*)nullptr, (const float2*)nullptr, hdev);
   } else if (!hyperball) {
     hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 0>), grid, block, 0, stream, items, prefix, n_items, h,
-                       (float*)nullptr, (const float2*)nullptr);
+                       (float*)nullptr, (const float2*)nullptr, hdev);
   } else {
     float* partial = scratch;
     float2* coef = (float2*)(scratch + (size_t)3 * total_chunks + ((total_chunks & 1) ? 1 : 0));
     hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 1>), grid, block, 0, stream, items, prefix, n_items, h,
-                       partial, (const float2*)nullptr);
-    hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), block, 0, stream, prefix, partial, h.lr, h.eps, coef);
+                       partial, (const float2*)nullptr, hdev);
+    hipLaunchKernelGGL(muonh_coef_kernel, dim3(n_items), block, 0, stream, prefix, partial, h.lr, h.eps, coef, hdev);
     hipLaunchKernelGGL((scalar_update_kernel<ALGO_ADAMW, 2>), grid, block, 0, stream, items, prefix, n_items, h,
-                       (float*)nullptr, (const float2*)coef);
+                       (float*)nullptr, (const float2*)coef, hdev);
   }
   return hipGetLastError();
 }

@@ -243,6 +243,12 @@ class Muon(Optimizer):
                         parameter's orientation (default; falls back to separate calls with a hook or a tight limit)
       ns_workspace_limit  upper bound in bytes for one batched Newton-Schulz workspace (larger classes
                           are processed in slices)
+      device_hyperparams  the weight-update kernels of every group read lr, lr*weight_decay, eps (and, for the AdamW /
+                          Lion groups, the betas' complements and bias corrections) from a small block in device
+                          memory instead of kernel arguments, so a ``step()`` captured in a HIP graph follows the
+                          schedule that the training loop writes into ``group["lr"]`` (pretrain.py:829-877): call
+                          ``sync_hyperparameters(advance_step=True)`` before each replay.  The momentum factor, the
+                          Newton-Schulz epsilon and the coefficient table stay kernel arguments.
     """
 
     def __init__(
@@ -267,6 +273,7 @@ class Muon(Optimizer):
         muonh_per_matrix: bool = False,
         ns_workspace_limit: int = 48 << 30,
         fuse_momentum: bool = True,
+        device_hyperparams: bool = False,
     ):
         if lr < 0.0:
             raise ValueError(f"Invalid learning rate: {lr}")
@@ -318,6 +325,8 @@ class Muon(Optimizer):
         self._muonh_per_matrix = muonh_per_matrix
         self._ns_workspace_limit = int(ns_workspace_limit)
         self._fuse_momentum = bool(fuse_momentum)
+        self._device_hyper = bool(device_hyperparams)
+        self._hyper_tables: Dict[int, _DeviceTable] = {}
         self._plans: Dict[int, Tuple[Tuple, _GroupPlan]] = {}
         self._scalar_plans: dict = {}
         #: when set to a list, every phase of a muon group step appends (name, start_event, stop_event)
@@ -332,6 +341,44 @@ class Muon(Optimizer):
         for p in params:
             self._hyperball_excluded.add(p)
 
+    # ------------------------------------------------------------------ hyper-parameters in device memory
+    def _group_device(self, group: dict) -> Optional[torch.device]:
+        for p in group["params"]:
+            return to_local([p])[0].device
+        return None
+
+    def _hyper_table(self, gi: int, group: dict) -> Optional[_DeviceTable]:
+        tab = self._hyper_tables.get(gi)
+        if tab is None:
+            device = self._group_device(group)
+            if device is None or device.type != "cuda":
+                return None
+            tab = _DeviceTable(_lib.HYPER.itemsize, device)
+            self._hyper_tables[gi] = tab
+        return tab
+
+    def _upload_group_hyper(self, gi: int, group: dict) -> None:
+        tab = self._hyper_table(gi, group)
+        if tab is None:
+            return
+        lr, wd = float(group["lr"]), float(group["weight_decay"])
+        rec = _lib.hyper_record(lr, lr * wd, float(group["epsilon"]), float(group["beta1"]), float(group["beta2"]),
+                                int(group["step"]), bool(group["cautious_wd"]))
+        with torch.cuda.device(tab.dev.device):
+            tab.upload(rec)
+
+    def sync_hyperparameters(self, advance_step: bool = False) -> None:
+        """With ``device_hyperparams``: copy the current hyper-parameters of every param group to the device block that
+        the kernels read (one small asynchronous copy per group on the current stream). ``step()`` does this itself
+        when it runs eagerly; a step that was captured in a HIP graph cannot, so call this before each replay, with
+        ``advance_step=True`` to count the replay as a step (``group["step"]``, the AdamW bias corrections)."""
+        if not self._device_hyper:
+            raise RuntimeError("sync_hyperparameters() needs Muon(..., device_hyperparams=True)")
+        for gi, group in enumerate(self.param_groups):
+            if advance_step:
+                group["step"] += 1
+            self._upload_group_hyper(gi, group)
+
     # ------------------------------------------------------------------ step
     @torch.no_grad()
     def step(self, closure=None):
@@ -340,26 +387,38 @@ class Muon(Optimizer):
             with torch.enable_grad():
                 loss = closure()
 
+        # a step that is being captured in a graph runs nothing now: its replays are counted, and their hyper-parameters
+        # uploaded, by sync_hyperparameters()
+        capturing = self._device_hyper and torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
         muon_groups, lion_groups, adamw_groups = [], [], []
         for gi, group in enumerate(self.param_groups):
-            group["step"] += 1
+            if not capturing:
+                group["step"] += 1
             algo = group["algorithm"]
             if algo == "muon":
                 muon_groups.append((gi, group))
             elif algo == "lion":
-                lion_groups.append(group)
+                lion_groups.append((gi, group))
             elif algo == "adamw":
-                adamw_groups.append(group)
+                adamw_groups.append((gi, group))
             else:
                 raise ValueError(f"Unknown algorithm: {algo}")
+            if self._device_hyper and not capturing:
+                self._upload_group_hyper(gi, group)
 
         for gi, group in muon_groups:
             self._muon_group_step(gi, group)
-        for group in lion_groups:
-            self._lion_group_step(group)
-        for group in adamw_groups:
-            self._adamw_group_step(group)
+        for gi, group in lion_groups:
+            self._lion_group_step(gi, group)
+        for gi, group in adamw_groups:
+            self._adamw_group_step(gi, group)
         return loss
+
+    def _hyper_ptr(self, gi: int, group: dict) -> Optional[int]:
+        if not self._device_hyper:
+            return None
+        tab = self._hyper_table(gi, group)
+        return None if tab is None else tab.dev.data_ptr()
 
     def _get_or_initialize_state(self, param: Tensor, algo: str) -> dict:
         state = self.state[param]
@@ -421,8 +480,17 @@ class Muon(Optimizer):
                 else:
                     self._orthogonalize_with_hook(plan, eps)
             # weight update                                                   (muon.py:598-650)
+            hyper = self._hyper_ptr(gi, group)
             with self._timed("update_muonh" if self.use_muonh else "update_plain"):
-                if self.use_muonh:
+                if hyper is not None and self.use_muonh:
+                    _lib.check(L.muon_update_muonh_dev(plan.post_tab.dev.data_ptr(), plan.post_prefix_dev.data_ptr(),
+                                                       len(plan.post_rows), plan.post_chunks, hyper,
+                                                       plan.scratch.data_ptr(), stream), "muon_update_muonh_dev")
+                elif hyper is not None:
+                    _lib.check(L.muon_update_plain_dev(plan.post_tab.dev.data_ptr(), plan.post_prefix_dev.data_ptr(),
+                                                       len(plan.post_rows), plan.post_chunks, hyper, stream),
+                               "muon_update_plain_dev")
+                elif self.use_muonh:
                     _lib.check(L.muon_update_muonh(plan.post_tab.dev.data_ptr(), plan.post_prefix_dev.data_ptr(),
                                                    len(plan.post_rows), plan.post_chunks, lr, lr * wd, eps,
                                                    int(cautious), plan.scratch.data_ptr(), stream),
@@ -495,7 +563,7 @@ class Muon(Optimizer):
             u.copy_(self._newton_schulz_func(x, epsilon=eps_t).reshape(p.shape))
 
     # ------------------------------------------------------------------ lion / adamw
-    def _lion_group_step(self, group: dict) -> None:
+    def _lion_group_step(self, gi: int, group: dict) -> None:
         params = [p for p in group["params"] if p.grad is not None]
         if not params:
             return
@@ -504,9 +572,9 @@ class Muon(Optimizer):
         scalar_opts.lion_update_foreach(
             to_local(params), grads, to_local(moms), float(group["lr"]),
             float(group["beta1"]), float(group["beta2"]), float(group["weight_decay"]), bool(group["cautious_wd"]),
-            key=("lion", tuple(id(p) for p in params)), cache=self._scalar_plans)
+            key=("lion", tuple(id(p) for p in params)), cache=self._scalar_plans, hyper_dev=self._hyper_ptr(gi, group))
 
-    def _adamw_group_step(self, group: dict) -> None:
+    def _adamw_group_step(self, gi: int, group: dict) -> None:
         params = [p for p in group["params"] if p.grad is not None]
         if not params:
             return
@@ -524,7 +592,8 @@ class Muon(Optimizer):
                 grads = [g if g.is_contiguous() else g.contiguous() for g in to_local([p.grad for p in plist])]
                 fn(to_local(plist), grads, to_local([s["momentum"] for s in states]),
                    to_local([s["variance"] for s in states]), *args,
-                   key=("adamw", tuple(id(p) for p in plist)), cache=self._scalar_plans)
+                   key=("adamw", tuple(id(p) for p in plist)), cache=self._scalar_plans,
+                   hyper_dev=self._hyper_ptr(gi, group))
 
 
 def zeropower_via_newtonschulz5(G: Tensor, epsilon: Union[float, Tensor] = 1e-7) -> Tensor:

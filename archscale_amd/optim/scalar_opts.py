@@ -53,7 +53,8 @@ _plans: Dict[Tuple, _ScalarPlan] = {}
 
 
 def _run(cache, key, algo: int, hyperball: bool, X: List[Tensor], G: List[Tensor], M: List[Tensor], V, lr: float, beta1: float,
-         beta2: float, weight_decay: float, step: int, epsilon: float, cautious_wd: bool) -> None:
+         beta2: float, weight_decay: float, step: int, epsilon: float, cautious_wd: bool,
+         hyper_dev: Optional[int] = None) -> None:
     if not X:
         return
     device = X[0].device
@@ -72,6 +73,12 @@ def _run(cache, key, algo: int, hyperball: bool, X: List[Tensor], G: List[Tensor
         cache[struct] = plan
     with torch.cuda.device(device):
         plan.refresh(X, G, M, V)
+        if hyper_dev is not None:   # hyper-parameters from a muon_hyper block in device memory (a captured step)
+            st = _lib.lib().muon_scalar_update_dev(
+                plan.table.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(X), plan.chunks, algo, int(hyperball),
+                hyper_dev, plan.scratch.data_ptr() if hyperball else 0, _lib.current_stream_ptr(device))
+            _lib.check(st, "muon_scalar_update_dev")
+            return
         st = _lib.lib().muon_scalar_update(
             plan.table.dev.data_ptr(), plan.prefix_dev.data_ptr(), len(X), plan.chunks, algo, int(hyperball),
             lr, beta1, beta2, lr * weight_decay, epsilon, max(int(step), 1), int(cautious_wd),
@@ -79,23 +86,24 @@ def _run(cache, key, algo: int, hyperball: bool, X: List[Tensor], G: List[Tensor
     _lib.check(st, "muon_scalar_update")
 
 
-def adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False, *, key=None, cache=None):
+def adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False, *, key=None, cache=None,
+                         hyper_dev=None):
     """AdamW with bias correction over a list of tensors (scalar_opts.py:118-198 of the reference)."""
     _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_ADAMW, False, X, G, M, V, lr, beta1, beta2, weight_decay, step,
-         epsilon, cautious_wd)
+         epsilon, cautious_wd, hyper_dev)
 
 
 def hyperball_adamw_update_foreach(X, G, M, V, lr, beta1, beta2, weight_decay, step, epsilon, cautious_wd=False, *,
-                                   key=None, cache=None):
+                                   key=None, cache=None, hyper_dev=None):
     """Adam direction applied on the hypersphere, per tensor (scalar_opts.py:254-377, 396-437 of the reference)."""
     _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_ADAMW, True, X, G, M, V, lr, beta1, beta2, weight_decay, step,
-         epsilon, cautious_wd)
+         epsilon, cautious_wd, hyper_dev)
 
 
-def lion_update_foreach(X, G, M, lr, beta1, beta2, weight_decay, cautious_wd=False, *, key=None, cache=None):
+def lion_update_foreach(X, G, M, lr, beta1, beta2, weight_decay, cautious_wd=False, *, key=None, cache=None, hyper_dev=None):
     """Lion over a list of tensors (scalar_opts.py:201-251 of the reference)."""
     _run(cache, key or tuple(id(x) for x in X), _lib.ALGO_LION, False, X, G, M, None, lr, beta1, beta2, weight_decay, 1, 0.0,
-         cautious_wd)
+         cautious_wd, hyper_dev)
 
 
 def release_plans() -> None:

@@ -220,6 +220,7 @@ def main():
     ap.add_argument("--seed", type=int, default=1236)
     ap.add_argument("--min-timed-seconds", type=float, default=2.0,
                     help="the block of --steps steps is repeated until the timed region is at least this long")
+    ap.add_argument("--dump-launches", action="store_true", help="(debug) every timed launch of the instrumented step on stderr")
     ap.add_argument("--other-configs", default="1,3,4,5",
                     help="comma-separated benchmark configurations reported beside the headline (empty: none)")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
@@ -268,6 +269,9 @@ def main():
     opt.step()
     torch.cuda.synchronize()
     recs = _lib.profile_collect()
+    if args.dump_launches:
+        for r in recs:
+            print(json.dumps({k: (round(v, 4) if isinstance(v, float) and k == "ms" else v) for k, v in r.items()}), file=sys.stderr)
     phases = {}
     for name, a, b in opt.phase_events:
         phases[name] = phases.get(name, 0.0) + a.elapsed_time(b)

@@ -264,6 +264,32 @@ int muon_scalar_update(const muon_scalar_item* items_dev, const int32_t* prefix_
                        int algo, int hyperball, float lr, float beta1, float beta2, float lr_wd, float eps, int step,
                        int cautious, float* scratch_dev, void* stream);
 
+/* ---- hyper-parameters from device memory ---------------------------------------------------------------------
+ * The training loop rewrites the learning rate (and, under batch ramp-up, weight decay and eps) of every param group
+ * before each step (pretrain.py:829-877), and the bias corrections of AdamW change with the step count.  Scalars that
+ * are kernel arguments are frozen into a captured HIP graph; the *_dev variants below read them from a muon_hyper block
+ * in DEVICE memory instead, which the caller refreshes with one small asynchronous copy before each replay, outside the
+ * graph.  Same kernels and same arithmetic as the by-value entry points (bit-identical results for equal values).
+ *   muon_update_plain_dev  uses lr, lr_wd, cautious           (replaces the scalars of muon_update_plain)
+ *   muon_update_muonh_dev  uses lr, lr_wd, eps, cautious      (muon_update_muonh)
+ *   muon_scalar_update_dev uses every field                    (muon_scalar_update; the host computes
+ *                          w1 = 1 - beta1, w2 = 1 - beta2 in float, bias1 = 1 - beta1^step and
+ *                          bias2_sqrt = sqrt(1 - beta2^step) in double, rounded to float)
+ */
+typedef struct muon_hyper {
+  float lr, lr_wd, eps;
+  float w1, w2;            /* 1 - beta1, 1 - beta2 */
+  float bias1, bias2_sqrt; /* 1 - beta1^step, sqrt(1 - beta2^step) */
+  int32_t cautious;
+} muon_hyper;
+
+int muon_update_plain_dev(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                          const muon_hyper* hyper_dev, void* stream);
+int muon_update_muonh_dev(const muon_post_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                          const muon_hyper* hyper_dev, float* scratch_dev, void* stream);
+int muon_scalar_update_dev(const muon_scalar_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks,
+                           int algo, int hyperball, const muon_hyper* hyper_dev, float* scratch_dev, void* stream);
+
 /* ---- MuonBall: spectral norm by power iteration, retraction and update ---------------------------------
  * muon_spectral_norm estimates the top singular value of every matrix of every shape class with the vector
  * sequence of power_iteration (emerging_optimizers/orthogonalized_optimizers/spectral_ball_utils.py:151-166:

@@ -50,7 +50,14 @@ def test_struct_layouts_and_constants_match_header():
         _fields_ = [("w", ctypes.c_void_p), ("u", ctypes.c_void_p), ("numel", ctypes.c_int64),
                     ("lr_ratio", ctypes.c_float), ("w_dtype", ctypes.c_int32)]
 
-    for cs, nd in ((Pre, _lib.PRE_ITEM), (Post, _lib.POST_ITEM)):
+    class Hyper(ctypes.Structure):
+        _fields_ = [(n, ctypes.c_float) for n in ("lr", "lr_wd", "eps", "w1", "w2", "bias1", "bias2_sqrt")] + [
+            ("cautious", ctypes.c_int32)]
+
+    m = re.search(r"typedef struct muon_hyper \{(.*?)\} muon_hyper;", text, re.S)
+    fields = re.findall(r"\b(\w+)\s*[,;]", re.sub(r"/\*.*?\*/", "", m.group(1), flags=re.S))
+    assert fields == [n for n, _ in Hyper._fields_]          # the header declares the fields in the binding's order
+    for cs, nd in ((Pre, _lib.PRE_ITEM), (Post, _lib.POST_ITEM), (Hyper, _lib.HYPER)):
         assert ctypes.sizeof(cs) == nd.itemsize
         for name, _ in cs._fields_:
             assert getattr(cs, name).offset == nd.fields[name][1]
@@ -71,6 +78,11 @@ def test_workspace_and_flops_queries_need_no_gpu():
     d2, s2, i2 = _lib.ns_flops(1, 512, 2048, 5, 1)
     assert i2 > i and d2 == d
     assert L.muon_muonh_scratch_floats(3, 10) >= 3 * 10 + 2 * 3
+    # the hyper-parameter record: derived fields as the by-value entry points compute them
+    rec = _lib.hyper_record(0.02, 0.02 * 0.1, 1e-8, 0.9, 0.95, 3, True)[0]
+    assert rec["w1"] == np.float32(1.0) - np.float32(0.9) and rec["cautious"] == 1
+    assert rec["bias1"] == np.float32(1.0 - float(np.float32(0.9)) ** 3)
+    assert rec["bias2_sqrt"] == np.float32((1.0 - float(np.float32(0.95)) ** 3) ** 0.5)
 
 
 def test_argument_errors_without_touching_the_gpu():

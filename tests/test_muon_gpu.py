@@ -481,3 +481,96 @@ def test_random_parameter_sets(gpu_device):
             assert torch.isfinite(p.detach().float()).all()
             assert _rel(p.detach(), xf) <= W_TOL, (case, tuple(p.shape))
             assert _rel(opt.state[p]["momentum"], mf) <= (1e-6 if wdtype == torch.float32 else 1e-2)
+
+
+def test_captured_step_follows_the_schedule(gpu_device):
+    """With device_hyperparams the weight-update kernels read lr, lr*wd, eps and the AdamW bias corrections from device
+    memory: a step captured ONCE follows a learning-rate schedule and the step count over its replays. Every replay is
+    checked bit for bit against an eager twin that gets the same values as kernel arguments (pretrain.py:829-877 rewrites
+    group["lr"] before every step)."""
+    from archscale_amd.optim.muon import Muon
+    shapes = [(128, 256), (256, 128), (2, 192, 64)]
+    g = torch.Generator().manual_seed(78)
+    W0 = [(torch.randn(*s, generator=g) * 0.02).to(torch.bfloat16) for s in shapes]
+    E0 = (torch.randn(300, 64, generator=g) * 0.02).to(torch.bfloat16)      # an AdamW matrix (hyperball), and a vector
+    V0 = torch.ones(64, dtype=torch.bfloat16)
+
+    def build(**kw):
+        mats = [torch.nn.Parameter(w.clone().to(gpu_device)) for w in W0]
+        emb, vec = torch.nn.Parameter(E0.clone().to(gpu_device)), torch.nn.Parameter(V0.clone().to(gpu_device))
+        groups = [dict(params=mats), dict(params=[emb, vec], algorithm="adamw", weight_decay=0.05)]
+        opt = Muon(groups, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True, use_muonh=True, cautious_wd=True, **kw)
+        return mats + [emb, vec], opt
+
+    pa, oa = build(device_hyperparams=True)
+    pb, ob = build()
+    all_shapes = shapes + [(300, 64), (64,)]
+    static_g = [torch.zeros_like(p) for p in pa]
+    for p, sg in zip(pa, static_g):
+        p.grad = sg
+
+    def new_grads(k):
+        gg = torch.Generator().manual_seed(2000 + k)
+        return [(torch.randn(*s, generator=gg) * 1e-3).to(torch.bfloat16).to(gpu_device) for s in all_shapes]
+
+    def schedule(k):
+        return 0.02 * (0.5 + 0.1 * k), 0.01 * (1 + k % 3)
+
+    def set_hyper(opt, k):
+        lr, wd = schedule(k)
+        for group in opt.param_groups:
+            group["lr"] = lr * (0.1 if group["algorithm"] == "adamw" else 1.0)
+            if group["algorithm"] == "muon":
+                group["weight_decay"] = wd
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for k in range(2):                                   # eager warm-up with the device block in use
+            for sg, gr in zip(static_g, new_grads(k)):
+                sg.copy_(gr)
+            set_hyper(oa, k)
+            oa.step()
+    torch.cuda.current_stream().wait_stream(side)
+    for k in range(2):
+        for p, gr in zip(pb, new_grads(k)):
+            p.grad = gr
+        set_hyper(ob, k)
+        ob.step()
+    torch.cuda.synchronize()
+    for a, b in zip(pa, pb):
+        assert torch.equal(a, b)                             # device block and kernel arguments: the same arithmetic
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        oa.step()
+    assert [grp["step"] for grp in oa.param_groups] == [2, 2]      # the capture itself is not a step
+    for k in range(2, 7):
+        for sg, gr in zip(static_g, new_grads(k)):
+            sg.copy_(gr)
+        set_hyper(oa, k)
+        oa.sync_hyperparameters(advance_step=True)
+        graph.replay()
+        for p, gr in zip(pb, new_grads(k)):
+            p.grad = gr
+        set_hyper(ob, k)
+        ob.step()
+        junk = torch.randn(128, 128, device=gpu_device) @ torch.randn(128, 128, device=gpu_device)   # eager work in between
+        torch.cuda.synchronize()
+        assert torch.isfinite(junk).all()
+        for a, b in zip(pa, pb):
+            assert torch.equal(a, b), k
+        assert [grp["step"] for grp in oa.param_groups] == [grp["step"] for grp in ob.param_groups]
+    # and the schedule really reached the kernels: a replay without the refresh repeats the last learning rate
+    before = [p.detach().clone() for p in pa]
+    for sg, gr in zip(static_g, new_grads(7)):
+        sg.copy_(gr)
+    graph.replay()
+    for p, gr in zip(pb, new_grads(7)):
+        p.grad = gr
+    set_hyper(ob, 7)
+    ob.step()
+    torch.cuda.synchronize()
+    assert not all(torch.equal(a, b) for a, b in zip(pa, pb))
+    assert not all(torch.equal(a, b) for a, b in zip(pa, before))
+    with pytest.raises(RuntimeError):
+        ob.sync_hyperparameters()
