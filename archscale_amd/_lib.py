@@ -29,6 +29,7 @@ NS_NO_GRAM_TAIL = 8
 NS_GRAM_TAIL = 16
 CHUNK_ELEMS = 8192
 NS_STATIC_SCRATCH_BYTES = 64 << 20
+STREAM_COPY, STREAM_READ, STREAM_MIX = 0, 1, 2
 E_STATIC_LIMIT = -4
 PROF_KEY_MOMENTUM_LAYOUT = 90000
 ABI_VERSION = 2
@@ -120,6 +121,8 @@ _SIGNATURES = {
         ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_void_p]),
     "muon_calibration_copy": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_calibration_stream": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                               ctypes.c_size_t, ctypes.c_void_p]),
     "muon_syrk_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 3),
     "muon_syrk": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,

@@ -941,6 +941,14 @@ int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void
   return (int)launch_calibration_copy(src_dev, dst_dev, bytes, (hipStream_t)stream);
 }
 
+int muon_calibration_stream(int mode, const void* a_dev, void* b_dev, void* c_dev, size_t bytes, void* stream) {
+  if (mode == MUON_STREAM_COPY) return muon_calibration_copy(a_dev, b_dev, bytes, stream);
+  if (mode != MUON_STREAM_READ && mode != MUON_STREAM_MIX) return MUON_E_ARG;
+  if (!a_dev || !b_dev || (bytes & 15) || ((uintptr_t)a_dev & 15) || ((uintptr_t)b_dev & 15)) return MUON_E_ARG;
+  if (mode == MUON_STREAM_MIX && (!c_dev || ((uintptr_t)c_dev & 15))) return MUON_E_ARG;
+  return (int)launch_calibration_stream(mode, a_dev, b_dev, c_dev, bytes, (hipStream_t)stream);
+}
+
 int muon_profile_begin(void) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
   g_prof.clear();

@@ -82,5 +82,7 @@ hipError_t launch_scalar_update(const ScalarItem* items, const int32_t* prefix, 
                                 const ScalarHyper* hdev = nullptr);
 
 hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+// mode 1: read a; mode 2: b <- a + b, c <- (a + b) ^ a (two reads, two writes)
+hipError_t launch_calibration_stream(int mode, const void* a, void* b, void* c, size_t bytes, hipStream_t stream);
 
 }  // namespace archscale

@@ -115,29 +115,38 @@ __device__ __forceinline__ void momentum_range(const PreItem& it, long begin, lo
                                                float* ss = nullptr) {
   const void* g = it.g; void* m = it.m; void* u = it.u;
   if (vec_ok) {
+    // every load of the chunk first, then the arithmetic and the stores: the stores may alias the loads as far as the
+    // compiler knows, and a load that waits for the previous trip's stores leaves the memory pipeline half empty
+    float gv[EW_TRIPS][8], mv[EW_TRIPS][8];
 #pragma unroll
     for (int t = 0; t < EW_TRIPS; ++t) {
       const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
       if (i < end) {
-        float gv[8], mv[8], uv[8];
-        Elem<GD>::load8(g, i, gv);
-        Elem<MD>::load8(m, i, mv);
+        Elem<GD>::load8(g, i, gv[t]);
+        Elem<MD>::load8(m, i, mv[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+        float uv[8];
         if (c.l2 != 0.f) {
           float wv[8];
           if (it.w_dtype == DT_BF16) Elem<DT_BF16>::load8(it.w, i, wv); else Elem<DT_F32>::load8(it.w, i, wv);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) gv[k] = Elem<GD>::round(gv[k] + c.l2 * wv[k]);
-          Elem<GD>::store8(const_cast<void*>(g), i, gv);
+          for (int k = 0; k < 8; ++k) gv[t][k] = Elem<GD>::round(gv[t][k] + c.l2 * wv[k]);
+          Elem<GD>::store8(const_cast<void*>(g), i, gv[t]);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-          const float gm = Elem<MD>::round(gv[k]);            // G cast to M's dtype (muon.py:666)
-          const float mn = Elem<MD>::round(fmaf(c.mm, mv[k], c.mg * gm));
-          mv[k] = mn;
+          const float gm = Elem<MD>::round(gv[t][k]);            // G cast to M's dtype (muon.py:666)
+          const float mn = Elem<MD>::round(fmaf(c.mm, mv[t][k], c.mg * gm));
+          mv[t][k] = mn;
           uv[k] = fmaf(c.um, mn, c.ug * gm);
           if (SS) { const float x = Elem<UD>::round(uv[k]); *ss += x * x; }
         }
-        Elem<MD>::store8(m, i, mv);
+        Elem<MD>::store8(m, i, mv[t]);
         Elem<UD>::store8(u, i, uv);
       }
     }
@@ -664,16 +673,22 @@ template <int WD, bool HAS_COEF>
 __device__ __forceinline__ void post_apply_range(const PostItem& it, long begin, long end, float lrwd, int cautious,
                                                  bool vec_ok, float alpha, float beta) {
   if (vec_ok) {
+    float x[EW_TRIPS][8], u[EW_TRIPS][8];   // all loads of the chunk before the first store (see momentum_range)
 #pragma unroll
     for (int t = 0; t < EW_TRIPS; ++t) {
       const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
       if (i < end) {
-        float x[8], u[8];
-        Elem<WD>::load8(it.w, i, x);
-        Elem<DT_BF16>::load8(it.u, i, u);
+        Elem<WD>::load8(it.w, i, x[t]);
+        Elem<DT_BF16>::load8(it.u, i, u[t]);
+      }
+    }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) x[k] = alpha * decayed(x[k], u[k], lrwd, cautious) + beta * u[k];
-        Elem<WD>::store8(it.w, i, x);
+    for (int t = 0; t < EW_TRIPS; ++t) {
+      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
+      if (i < end) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[t][k] = alpha * decayed(x[t][k], u[t][k], lrwd, cautious) + beta * u[t][k];
+        Elem<WD>::store8(it.w, i, x[t]);
       }
     }
   } else {
@@ -883,6 +898,57 @@ calibration_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, 
       if (i < n16) stream_store16(dst + i, v[u]);
     }
   }
+}
+
+// The same access pattern as a pure read (mode 1: the words are folded into a checksum that is written only if it
+// equals a value the fill pattern never produces) and as the momentum kernel's mix of two reads and two writes
+// (mode 2: b <- a + b, c <- (a + b) xor a): the rates these reach are what an HBM-bound kernel of that mix can reach.
+template <int MODE>
+__global__ void __launch_bounds__(256)
+calibration_stream_kernel(const u32x4* __restrict__ a, u32x4* __restrict__ b, u32x4* __restrict__ c, long n16) {
+  const long stride = (long)gridDim.x * blockDim.x * CAL_UNROLL;
+  uint32_t fold = 0;
+  for (long base = (long)blockIdx.x * CAL_UNROLL * blockDim.x + threadIdx.x; base < n16; base += stride) {
+    u32x4 va[CAL_UNROLL], vb[CAL_UNROLL];
+#pragma unroll
+    for (int u = 0; u < CAL_UNROLL; ++u) {
+      const long i = base + (long)u * blockDim.x;
+      if (i < n16) {
+        va[u] = stream_load16(a + i);
+        if (MODE == 2) vb[u] = stream_load16(b + i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < CAL_UNROLL; ++u) {
+      const long i = base + (long)u * blockDim.x;
+      if (i < n16) {
+        if (MODE == 1) {
+          fold ^= va[u].x ^ va[u].y ^ va[u].z ^ va[u].w;
+        } else {
+          const u32x4 sum = va[u] + vb[u];
+          stream_store16(b + i, sum);
+          stream_store16(c + i, sum ^ va[u]);
+        }
+      }
+    }
+  }
+  if (MODE == 1 && fold == 0x9e3779b9u) ((uint32_t*)b)[0] = fold;
+}
+
+hipError_t launch_calibration_stream(int mode, const void* a, void* b, void* c, size_t bytes, hipStream_t stream) {
+  const long n16 = (long)(bytes / 16);
+  if (n16 <= 0) return hipSuccess;
+  long blocks = (n16 + 256 * CAL_UNROLL - 1) / (256 * CAL_UNROLL);
+  if (blocks > (1L << 20)) blocks = 1L << 20;
+  if (mode == 1)
+    hipLaunchKernelGGL(calibration_stream_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, (const u32x4*)a, (u32x4*)b,
+                       (u32x4*)c, n16);
+  else if (mode == 2)
+    hipLaunchKernelGGL(calibration_stream_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, (const u32x4*)a, (u32x4*)b,
+                       (u32x4*)c, n16);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
 }
 
 hipError_t launch_calibration_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {

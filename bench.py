@@ -288,6 +288,19 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # what the memory delivers to plain streaming kernels of known size on this GPU, right now: read-only, copy, and
+    # the two-read / two-write mix of the fused momentum kernel (the HBM-bound kernels are reported beside these)
+    yard = {}
+    if cal_bytes:
+        bufs = [torch.empty(cal_bytes, dtype=torch.uint8, device=dev).fill_(k + 1) for k in range(3)]
+        for name, mode, moved in (("read", _lib.STREAM_READ, 1), ("copy", _lib.STREAM_COPY, 2), ("mix_2r2w", _lib.STREAM_MIX, 4)):
+            fn = lambda: _lib.check(_lib.lib().muon_calibration_stream(mode, bufs[0].data_ptr(), bufs[1].data_ptr(),
+                                                                       bufs[2].data_ptr(), cal_bytes,
+                                                                       _lib.current_stream_ptr(dev)), "muon_calibration_stream")
+            gbs = moved * cal_bytes / _time_calls(fn, 10) / 1e6
+            yard[name] = {"GB/s": round(gbs), "frac": round(gbs / HBM_PEAK_GBS, 3)}
+        del bufs
+
     shapes = [tuple(p.shape) for p in params]
     n_elem = sum(p.numel() for p in params)
     f_dense = sum(dense_flops(s) for s in shapes)
@@ -393,6 +406,7 @@ def main():
         "kernel_fracs": kernel_fracs,
         "kernels": kernels,
         "hbm_kernels": hbm,
+        "hbm_yardsticks": yard,
         "phases_ms": {k: round(v, 3) for k, v in phases.items()},
         "calibration_copy_bytes": cal_bytes,
     }

@@ -160,6 +160,16 @@ int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algori
  * reference: a copy of known size is the yardstick that scales the HBM byte counters of a profiling run. */
 int muon_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream);
 
+/* Streaming yardsticks with the access pattern of the copy above (no counterpart in the reference): what this GPU's
+ * memory delivers to a kernel that only reads (MUON_STREAM_READ: `bytes` of a; b receives nothing but must be valid), that
+ * copies (MUON_STREAM_COPY: b <- a) or that has the fused momentum kernel's mix of two reads and two writes
+ * (MUON_STREAM_MIX: b <- a + b, c <- (a + b) xor a, as 32-bit words).  The rates of the HBM-bound kernels are reported
+ * beside these.  All buffers `bytes` long (a multiple of 16), 16-byte aligned; c_dev only for MUON_STREAM_MIX. */
+#define MUON_STREAM_COPY 0
+#define MUON_STREAM_READ 1
+#define MUON_STREAM_MIX 2
+int muon_calibration_stream(int mode, const void* a_dev, void* b_dev, void* c_dev, size_t bytes, void* stream);
+
 /* ---- single products on caller tensors ------------------------------------------------------
  * D = alpha * A A^T + beta * C, A [batch] n x k (bf16, row-major, ld lda), C symmetric n x n or NULL, D n x n,
  * both triangles written.  Replaces ns_line_1 / ns_line_2 (newton_schulz_triton.py:142-178, 269-310) and

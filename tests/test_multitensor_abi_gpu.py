@@ -104,3 +104,32 @@ def test_argument_errors_do_not_launch(gpu_device):
     assert L.muon_update_muonh(0, 0, 1, 1, 0.1, 0.0, 1e-8, 0, 0, 0) < 0
     assert L.muon_momentum(0, 0, 0, 0, 0.9, 1.0, 0.9, 1.0, 0.0, 0) == 0      # nothing to do
     torch.cuda.synchronize()
+
+
+def test_streaming_yardsticks(gpu_device):
+    """muon_calibration_stream: the copy, the read-only pass and the two-read / two-write mix do what the header says
+    (word-wise, on sizes that are and are not a multiple of a block's piece)."""
+    import numpy as np
+    from archscale_amd import _lib
+    L = _lib.lib()
+    stream = _lib.current_stream_ptr(gpu_device)
+    for n_words in (4, 4 * 1024 * 4, 4 * (3 * 1024 + 17)):
+        rng = np.random.default_rng(n_words)
+        a = torch.from_numpy(rng.integers(0, 2 ** 31, n_words, dtype=np.int64).astype(np.int32)).to(gpu_device)
+        b = torch.from_numpy(rng.integers(0, 2 ** 31, n_words, dtype=np.int64).astype(np.int32)).to(gpu_device)
+        c = torch.zeros_like(a)
+        a0, b0 = a.clone(), b.clone()
+        nbytes = 4 * n_words
+        assert L.muon_calibration_stream(_lib.STREAM_READ, a.data_ptr(), b.data_ptr(), 0, nbytes, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(a, a0) and torch.equal(b, b0)
+        assert L.muon_calibration_stream(_lib.STREAM_MIX, a.data_ptr(), b.data_ptr(), c.data_ptr(), nbytes, stream) == 0
+        torch.cuda.synchronize()
+        total = a0 + b0                     # int32 wrap-around = the kernel's unsigned 32-bit sum
+        assert torch.equal(b, total) and torch.equal(c, total ^ a0) and torch.equal(a, a0)
+        assert L.muon_calibration_stream(_lib.STREAM_COPY, a.data_ptr(), c.data_ptr(), 0, nbytes, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(c, a0)
+    assert L.muon_calibration_stream(7, a.data_ptr(), b.data_ptr(), c.data_ptr(), 16, stream) == -1
+    assert L.muon_calibration_stream(_lib.STREAM_MIX, a.data_ptr(), b.data_ptr(), 0, 16, stream) == -1
+    assert L.muon_calibration_stream(_lib.STREAM_READ, a.data_ptr(), b.data_ptr(), 0, 12, stream) == -1
