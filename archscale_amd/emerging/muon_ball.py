@@ -27,9 +27,11 @@ from torch.optim.optimizer import ParamsT
 from .. import _lib
 from ..optim import newton_schulz_hip as ns
 from ..optim.muon import _DeviceTable
+from ..optim.opt_utils import to_local
 from .mixin import WeightDecayT, weight_decay_terms
 from .orthogonalized_optimizer import OrthogonalizedOptimizer, _Plan
-from .spectral_ball_utils import compute_target_radius, get_spectral_ball_scale_factor, msign_schedule
+from .spectral_ball_utils import (compute_target_radius, get_spectral_ball_scale_factor, msign, msign_schedule,
+                                  spectral_norm)
 
 __all__ = ["MuonBall"]
 
@@ -465,8 +467,62 @@ class MuonBall(OrthogonalizedOptimizer):
             self.retract_bias_dict[key] = bias
             self.spectral_norm_dict[key] = s
 
+    def _compute_component_update(self, W: torch.Tensor, M: torch.Tensor, tp_group: Any = None,
+                                  partition_dim: Optional[int] = None, current_lr: Optional[float] = None,
+                                  param_name: Optional[str] = None, component_label: Optional[str] = None) -> torch.Tensor:
+        """One matrix (muon_ball.py:301-352): spectral norm by power iteration, retraction of ``W`` IN PLACE, then
+        ``scale * msign(M)``. ``W`` and ``M`` may be views into a parameter and its momentum (transposed ones included).
+        Hard retraction reads nothing back to the host; the dynamic mode reads sigma for its logging dictionaries, as the
+        reference does."""
+        if tp_group is not None and tp_group.size() > 1:
+            raise NotImplementedError("MuonBall on MI355X runs on one GPU: tensor-parallel groups must have one rank")
+        R = compute_target_radius(tuple(W.shape), self.radius_mode)
+        sigma = spectral_norm(W, self.power_iteration_steps)            # 0-d fp32 device tensor
+        if self.retract_mode == "hard":
+            W.mul_((R / (sigma.clamp_min(0.0) + 1e-8)).to(W.dtype))
+        else:
+            bias_t = torch.where(sigma > R, -1.0, 1.0)
+            step = self.retract_alpha * current_lr if current_lr is not None else self.retract_alpha
+            W.mul_((1.0 + step * bias_t).to(W.dtype))
+            if param_name and component_label:
+                self.retract_bias_dict[f"{param_name}.{component_label}"] = float(bias_t.item())
+                self.spectral_norm_dict[f"{param_name}.{component_label}"] = float(sigma.item())
+        phi = msign(M if M.dtype == torch.float32 else M.to(torch.float32), self.msign_steps)
+        return phi * get_spectral_ball_scale_factor(W.shape[0], W.shape[1], mode=self.scale_mode)
+
+    @torch.no_grad()
     def orthogonalize(self, p: torch.Tensor, grad: torch.Tensor, **kwargs: Any) -> torch.Tensor:
-        raise NotImplementedError("MuonBall.step() orthogonalises all pieces of a param group in batched device calls")
+        """The reference's public per-tensor entry (muon_ball.py:354-636): retracts ``p`` (every piece of a fused
+        parameter on its own) in place and returns the update direction shaped like ``p``, to be applied as
+        ``p.add_(update, alpha=-lr)``. ``grad`` is the momentum-processed gradient; ``lr`` comes in through ``kwargs``.
+        ``step()`` does not go through here (it runs every piece of a param group in batched device calls); this is for
+        callers and subclasses that use the reference's per-tensor contract. As in the reference, the QKV "component"
+        layout works on gathered copies, so the parameter itself is not retracted in that mode."""
+        lr = kwargs.get("lr", None)
+        t = to_local([p])[0]
+        g = to_local([grad])[0]
+        _lib.require_cuda(t, "a MuonBall parameter")
+        if not t.is_contiguous() or not g.is_contiguous() or g.shape != t.shape:
+            raise ValueError("parameter and gradient must be contiguous and of one shape")
+        name = getattr(p, "param_name", None)
+        update = torch.empty(t.shape, dtype=torch.bfloat16, device=t.device)
+        for pc in self._pieces_of(0, p, t):
+            if pc.gather is not None:
+                groups, ssum, row_off, part = pc.gather
+                sl = (slice(None), slice(row_off, row_off + part))
+                W = t.view(groups, ssum, pc.cols)[sl].reshape(-1, pc.cols)         # a copy, like the reference's reshape
+                M = g.view(groups, ssum, pc.cols)[sl].reshape(-1, pc.cols)
+                U = self._compute_component_update(W, M, None, None, lr, name, pc.label)
+                update.view(groups, ssum, pc.cols)[sl] = U.view(groups, part, pc.cols)
+                continue
+            W = torch.as_strided(t, (pc.rows, pc.cols), (pc.ld, 1), t.storage_offset() + pc.off)
+            M = torch.as_strided(g, (pc.rows, pc.cols), (pc.ld, 1), g.storage_offset() + pc.off)
+            out = torch.as_strided(update, (pc.rows, pc.cols), (pc.ld, 1), pc.off)
+            if pc.transposed:
+                out.copy_(self._compute_component_update(W.t(), M.t(), None, None, lr, name, pc.label).t())
+            else:
+                out.copy_(self._compute_component_update(W, M, None, None, lr, name, pc.label))
+        return update
 
     def get_retract_bias_dict(self):
         if self.retract_mode == "hard" or not self.retract_bias_dict:

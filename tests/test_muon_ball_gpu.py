@@ -356,3 +356,55 @@ def test_fused_momentum_matches_separate_calls(gpu_device):
     for a, b, m1, m2, w in zip(wf, ws, mf, ms, w0):
         assert rel(m1, m2) <= 2e-3
         assert rel(a - w, b - w) <= 1e-2
+
+
+@pytest.mark.parametrize("case", ["plain", "fc1", "qkv_group", "qkv_component", "moe1_split", "moe2"])
+@pytest.mark.parametrize("retract_mode", ["hard", "dynamic"])
+def test_orthogonalize_per_tensor(gpu_device, case, retract_mode):
+    """MuonBall.orthogonalize(p, grad, lr=...): the reference's per-tensor entry (muon_ball.py:354-636) retracts the
+    parameter (piece by piece) in place and returns the update; against the oracle's restatement of the same method."""
+    from archscale_amd.emerging import MuonBall
+    kw = dict(lr=0.02, momentum_beta=0.9, weight_decay=0.0, power_iteration_steps=8, msign_steps=5, retract_mode=retract_mode)
+    attrs, split, shape, name = {}, None, (96, 80), "attn.w"
+    if case == "fc1":
+        kw.update(split_fc1=True, is_fc1_fn=lambda p: True, fc1_split_shapes=(48, 48))
+        split = {"kind": "fc1", "shapes": (48, 48)}
+    elif case.startswith("qkv"):
+        shape, mode = (128, 80), case.split("_")[1]
+        kw.update(split_qkv=True, is_qkv_fn=lambda p: True, qkv_split_shapes=(32, 16, 16), qkv_split_mode=mode)
+        split = {"kind": "qkv", "shapes": (32, 16, 16), "mode": mode}
+    elif case == "moe1_split":
+        shape, name = (80, 192), "mlp.experts.weight1"
+        kw.update(split_moe_experts=True, is_grouped_moe_fn=lambda p: True, split_fc1=True)
+        attrs = dict(num_local_experts=3, is_gated=True)
+        split = {"kind": "moe1", "experts": 3, "gated": True, "split_fc1": True}
+    elif case == "moe2":
+        shape, name = (192, 80), "mlp.experts.weight2"
+        kw.update(split_moe_experts=True, is_grouped_moe_fn=lambda p: True)
+        attrs = dict(num_local_experts=4)
+        split = {"kind": "moe2", "experts": 4}
+    g = torch.Generator().manual_seed(23)
+    W0 = torch.randn(*shape, generator=g) * 0.05
+    M0 = torch.randn(*shape, generator=g) * 1e-2
+    p = _named(W0.clone().to(gpu_device), name, **attrs)
+    opt = MuonBall([p], **kw)
+    upd = opt.orthogonalize(p, M0.clone().to(gpu_device), lr=0.02)
+    torch.cuda.synchronize()
+    assert upd.shape == p.shape and upd.dtype == torch.bfloat16
+    x = W0.clone()
+    want = B.orthogonalize(x, M0.clone(), lr=0.02, split=split, radius_mode="spectral_mup", scale_mode="align_adamw_rms",
+                           power_iteration_steps=8, msign_steps=5, retract_mode=retract_mode, retract_alpha=0.05,
+                           ns_storage="fp32", sigma_fn=B.power_iteration_fp64)
+    assert _rel(upd, want) <= 1e-2, case
+    assert _rel(p.detach(), x) <= 5e-3, case                      # the retraction reached the parameter (fp32 weights)
+    if case != "qkv_component":
+        assert not torch.equal(p.detach().cpu(), W0)
+    else:
+        assert torch.equal(p.detach().cpu(), W0)                 # gathered copies: the parameter is not retracted, as in the reference
+    if retract_mode == "dynamic":
+        assert (len(opt.retract_bias_dict) > 0) == (case != "plain")   # logged per labelled component, like the reference
+    # applying it the way the base class does is one step of the optimizer
+    with torch.no_grad():
+        p.add_(upd.to(p.dtype), alpha=-0.02)
+    x.add_(want, alpha=-0.02)
+    assert _rel(p.detach(), x) <= W_TOL
