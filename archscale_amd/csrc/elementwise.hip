@@ -807,25 +807,39 @@ scalar_update_kernel(const ScalarItem* __restrict__ items, const int32_t* __rest
   if (PHASE == 2) { const float2 c = coef[ii]; alpha = c.x; beta = c.y; }
   float s[3] = {0.f, 0.f, 0.f};
   if (vec_ok) {
+    // two trips at a time: every load of the pair before its first store (the stores may alias the loads as far as
+    // the compiler knows, and a load that waits for the previous trip's stores leaves the memory pipeline half empty)
+    // (plain AdamW moves four arrays per element and is faster one trip at a time: 5.0 against 4.6 TB/s)
+    constexpr int PAIR = (ALGO == ALGO_ADAMW && PHASE == 0) ? 1 : 2;
+    static_assert(EW_TRIPS % PAIR == 0, "trips come in pairs");
 #pragma unroll
-    for (int t = 0; t < EW_TRIPS; ++t) {
-      const long i = begin + ((long)t * EW_THREADS + threadIdx.x) * EW_VEC;
-      if (i < end) {
-        float x[8], g[8], m[8], v[8];
-        load8_rt(it.w, it.w_dtype, i, x);
-        load8_rt(it.m, it.m_dtype, i, m);
-        if (PHASE != 2) load8_rt(it.g, it.g_dtype, i, g);
-        if (has_v) load8_rt(it.v, it.v_dtype, i, v);
+    for (int t0 = 0; t0 < EW_TRIPS; t0 += PAIR) {
+      float x[PAIR][8], g[PAIR][8], m[PAIR][8], v[PAIR][8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          if (PHASE == 2) g[k] = 0.f;
-          if (!has_v) v[k] = 0.f;
-          x[k] = scalar_elem<ALGO, PHASE>(x[k], g[k], m[k], v[k], h, it.m_dtype, it.v_dtype, alpha, beta, s);
+      for (int u = 0; u < PAIR; ++u) {
+        const long i = begin + ((long)(t0 + u) * EW_THREADS + threadIdx.x) * EW_VEC;
+        if (i < end) {
+          load8_rt(it.w, it.w_dtype, i, x[u]);
+          load8_rt(it.m, it.m_dtype, i, m[u]);
+          if (PHASE != 2) load8_rt(it.g, it.g_dtype, i, g[u]);
+          if (has_v) load8_rt(it.v, it.v_dtype, i, v[u]);
         }
-        if (PHASE != 1) store8_rt(it.w, it.w_dtype, i, x);
-        if (PHASE != 2) {
-          store8_rt(it.m, it.m_dtype, i, m);
-          if (has_v) store8_rt(it.v, it.v_dtype, i, v);
+      }
+#pragma unroll
+      for (int u = 0; u < PAIR; ++u) {
+        const long i = begin + ((long)(t0 + u) * EW_THREADS + threadIdx.x) * EW_VEC;
+        if (i < end) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            if (PHASE == 2) g[u][k] = 0.f;
+            if (!has_v) v[u][k] = 0.f;
+            x[u][k] = scalar_elem<ALGO, PHASE>(x[u][k], g[u][k], m[u][k], v[u][k], h, it.m_dtype, it.v_dtype, alpha, beta, s);
+          }
+          if (PHASE != 1) store8_rt(it.w, it.w_dtype, i, x[u]);
+          if (PHASE != 2) {
+            store8_rt(it.m, it.m_dtype, i, m[u]);
+            if (has_v) store8_rt(it.v, it.v_dtype, i, v[u]);
+          }
         }
       }
     }
