@@ -416,7 +416,10 @@ def main():
         del opt, params, grads, p, g
         _lib.release_workspaces()
         torch.cuda.empty_cache()
-        out["other_configs"] = other_configs(dev, which)
+        try:
+            out["other_configs"] = other_configs(dev, which)
+        except Exception as e:   # the headline above stands on its own
+            out["other_configs"] = {"error": f"{type(e).__name__}: {e}"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.coeffs, args.seed)
     print(json.dumps(out))
