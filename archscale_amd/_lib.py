@@ -150,6 +150,9 @@ _SIGNATURES = {
     "muon_spectral_norm_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(SnProblem), ctypes.c_int]),
     "muon_spectral_norm": (ctypes.c_int, [
         ctypes.POINTER(SnProblem), ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "muon_power_iteration": (ctypes.c_int, [
+        ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_ball_apply": (ctypes.c_int, [
         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int,
         ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p]),

@@ -798,10 +798,35 @@ size_t muon_spectral_norm_workspace_bytes(const muon_sn_problem* problems_host, 
   return total;
 }
 
+namespace {
+int spectral_norm_impl(const muon_sn_problem* problems_host, int n_problems, int steps, void* ws_dev, size_t ws_bytes,
+                       void* stream_, float* short_out, float* long_out);
+}
+
 int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int steps, void* ws_dev, size_t ws_bytes,
-                       void* stream_) {
+                       void* stream) {
+  return spectral_norm_impl(problems_host, n_problems, steps, ws_dev, ws_bytes, stream, nullptr, nullptr);
+}
+
+int muon_power_iteration(const void* const* w_ptrs_host, int dtype, int ld, int batch, int rows, int cols, int steps,
+                         float* sigma_out_dev, float* u_out_dev, float* v_out_dev, void* ws_dev, size_t ws_bytes,
+                         void* stream) {
+  if (!u_out_dev || !v_out_dev) return MUON_E_ARG;
+  muon_sn_problem q = {};
+  q.w_ptrs = w_ptrs_host; q.sigma_out = sigma_out_dev;
+  q.dtype = dtype; q.ld = ld; q.batch = batch; q.rows = rows; q.cols = cols; q.flags = 0;
+  // the short-side vector is u for a wide matrix and v for a tall one
+  const bool tall = rows > cols;
+  return spectral_norm_impl(&q, 1, steps, ws_dev, ws_bytes, stream, tall ? v_out_dev : u_out_dev,
+                            tall ? u_out_dev : v_out_dev);
+}
+
+namespace {
+int spectral_norm_impl(const muon_sn_problem* problems_host, int n_problems, int steps, void* ws_dev, size_t ws_bytes,
+                       void* stream_, float* short_out, float* long_out) {
   hipStream_t stream = (hipStream_t)stream_;
   if (!problems_host || n_problems <= 0 || steps < 1 || !ws_dev) return MUON_E_ARG;
+  if ((short_out || long_out) && (n_problems != 1 || !short_out || !long_out)) return MUON_E_ARG;
   if ((uintptr_t)ws_dev & 255) return MUON_E_WORKSPACE;
   // tall: the matrix meant (after MUON_SN_TRANSPOSED) has more rows than columns; use_t: its short-side-first copy is
   // the transpose of the stored block
@@ -923,9 +948,21 @@ int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int
       return st;
   }
   // the rounds: every application of G (or of a power of it) is one launch over all classes
-  if ((st = for_class_chunks([&](const SnParams& sp) { return launch_spectral_iterate(sp, steps, stream); })) != 0) return st;
+  int final_src[2] = {0, 0};
+  SnParams last = {};
+  if ((st = for_class_chunks([&](const SnParams& sp) {
+         last = sp;
+         return launch_spectral_iterate(sp, steps, stream, final_src);
+       })) != 0)
+    return st;
+  if (short_out) {   // one problem, one class: its singular vectors from the iterates that are still in the workspace
+    const SnClass& c = last.c[0];
+    const int L = pr[0].sp.pl.n;
+    if ((e = launch_spectral_vectors(c, L, final_src[c.tall ? 1 : 0], short_out, long_out, stream)) != hipSuccess) return (int)e;
+  }
   return 0;
 }
+}  // namespace
 
 int muon_ball_apply(const muon_ball_item* items_dev, const int32_t* prefix_dev, int n_items, int total_chunks, float lr,
                     float decay, int retract_mode, float retract_step, float* log_out_dev, void* stream) {

@@ -44,7 +44,14 @@ hipError_t launch_spectral_xscale(const SnParams& sp, hipStream_t stream);
 
 // init + the applications of G that `steps` rounds stand for (`steps` for wide matrices, `steps + 1` for tall ones, the
 // last one always G itself; the others G^4, G^2 or G as far as the class has them) + final
-hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t stream);
+// final_src (optional, two ints): which of the two z buffers holds the last iterate of the wide / of the tall classes
+hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t stream, int* final_src = nullptr);
+
+// after launch_spectral_iterate, for one class: short_out[b][d] = the short-side singular vector (unnormalised: u of a
+// wide matrix, v of a tall one), long_out[b][L] = X^T times the iterate before the last (v of a wide matrix, u of a
+// tall one, unnormalised); L = the true long extent
+hipError_t launch_spectral_vectors(const SnClass& c, int L, int src_final, float* short_out, float* long_out,
+                                   hipStream_t stream);
 
 hipError_t launch_ball_apply(const muon_ball_item* items, const int32_t* prefix, int n_items, int total_chunks, float lr,
                              float decay, int retract_mode, float retract_step, float* log_out, hipStream_t stream);

@@ -23,6 +23,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "spectral.h"
 
 namespace archscale {
@@ -213,7 +215,52 @@ hipError_t launch_spectral_xscale(const SnParams& sp, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t stream) {
+// The vectors of a finished iteration of ONE class: short_out[b][0..d) = z_short[b] and long_out[b][0..L) = X_b^T z_prev[b]
+// (X_b: d_p x L_p, zero padded; one lane owns 8 consecutive columns and walks down the rows)
+__global__ void __launch_bounds__(256)
+sn_vectors_kernel(const uint16_t* __restrict__ X, const float* __restrict__ z_prev, const float* __restrict__ z_short,
+                  float* __restrict__ short_out, float* __restrict__ long_out, int d, int d_p, int L, int L_p) {
+  const int b = blockIdx.y;
+  const long t = (long)blockIdx.x * 256 + threadIdx.x;
+  if (t < d) short_out[(size_t)b * d + t] = z_short[(size_t)b * d_p + t];
+  const long j0 = t * 8;
+  if (j0 >= L_p) return;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const uint16_t* col = X + (size_t)b * d_p * L_p + j0;
+  const float* zp = z_prev + (size_t)b * d_p;
+  for (int i = 0; i < d; ++i) {
+    const uint4 r = *(const uint4*)(col + (size_t)i * L_p);
+    const float zi = zp[i];
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      acc[2 * k] += bf2f_((uint16_t)(w[k] & 0xffff)) * zi;
+      acc[2 * k + 1] += bf2f_((uint16_t)(w[k] >> 16)) * zi;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k)
+    if (j0 + k < L) long_out[(size_t)b * L + j0 + k] = acc[k];
+}
+
+hipError_t launch_spectral_vectors(const SnClass& c, int L, int src_final, float* short_out, float* long_out,
+                                   hipStream_t stream) {
+  if (!short_out || !long_out || c.batch <= 0 || c.batch > 65535 || c.d <= 0 || c.d > c.d_p || L <= 0 || L > c.L_p ||
+      c.L_p % 8 || (src_final != 0 && src_final != 1))
+    return hipErrorInvalidValue;
+  const float* z_final = c.z + (size_t)src_final * c.batch * c.d_p;
+  const float* z_prev = c.z + (size_t)(src_final ^ 1) * c.batch * c.d_p;
+  // wide matrices (G = W W^T): the short vector is the LAST iterate, G^steps W 1 (the reference's u); tall ones
+  // (G = W^T W): the one before it, G^steps 1 (the reference's v); the long vector is X^T times the one before the last
+  const float* z_short = c.tall ? z_prev : z_final;
+  const long lanes = std::max((long)c.L_p / 8, (long)c.d);
+  const unsigned blocks = (unsigned)((lanes + 255) / 256);
+  hipLaunchKernelGGL(sn_vectors_kernel, dim3(blocks, c.batch), dim3(256), 0, stream, (const uint16_t*)c.X, z_prev, z_short,
+                     short_out, long_out, c.d, c.d_p, L, c.L_p);
+  return hipGetLastError();
+}
+
+hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t stream, int* final_src) {
   if (sp.n < 1 || sp.n > SN_MAX_CLASSES || steps < 1) return hipErrorInvalidValue;
   const int blocks = sp.blk_start[sp.n];
   int matrices = 0;
@@ -256,6 +303,7 @@ hipError_t launch_spectral_iterate(const SnParams& sp, int steps, hipStream_t st
     if (w1 >= 0) src[1] ^= 1;
   }
   hipLaunchKernelGGL(sn_final_kernel, dim3(matrices), dim3(64), 0, stream, sp, src[0], src[1]);
+  if (final_src) { final_src[0] = src[0]; final_src[1] = src[1]; }
   return hipGetLastError();
 }
 

@@ -78,16 +78,44 @@ def spectral_norm(w: torch.Tensor, steps: int = 50) -> torch.Tensor:
 
 @torch.no_grad()
 def power_iteration(w: torch.Tensor, steps: int = 50, eps: float = 1e-20):
-    """(sigma, u, v) like spectral_ball_utils.py:151-166 of the reference. ``sigma`` comes from the HIP path
-    (:func:`spectral_norm`); the singular vectors, which MuonBall does not use, are recovered with plain matrix-vector
-    products (``eps`` is unused, as in the reference)."""
-    sigma = spectral_norm(w, steps)
-    wb = w.to(torch.bfloat16)
-    v = torch.ones_like(wb[..., :1, :].transpose(-2, -1))
-    for _ in range(steps):
-        v = torch.nn.functional.normalize(wb.transpose(-2, -1) @ (wb @ v), dim=-2)
-    u = torch.nn.functional.normalize(wb @ v, dim=-2)
-    return sigma, u, v
+    """(sigma, u, v) like spectral_ball_utils.py:151-166 of the reference: ``sigma`` fp32 of shape ``w.shape[:-2]``,
+    ``u`` ``[..., rows, 1]`` and ``v`` ``[..., cols, 1]`` unit vectors in bf16, all from the HIP path
+    (``muon_power_iteration``: the vector sequence runs on the Gram matrix of the short side; the short-side vector is
+    its last iterate, the long-side one a single pass over the matrix). ``eps`` is unused, as in the reference."""
+    import ctypes
+
+    from .. import _lib
+    if w.ndim < 2:
+        raise ValueError("Input tensor must have at least 2 dimensions.")
+    if steps < 1:
+        raise ValueError(f"steps must be at least 1, got {steps}")
+    _lib.require_cuda(w, "power_iteration input")
+    if w.dtype not in (torch.bfloat16, torch.float32):
+        w = w.to(torch.float32)
+    rows, cols = w.shape[-2:]
+    mats = w.reshape(-1, rows, cols)
+    if mats.stride(-1) != 1 or mats.stride(-2) < cols:
+        mats = mats.contiguous()
+    batch = mats.shape[0]
+    sigma = torch.empty(batch, dtype=torch.float32, device=w.device)
+    u = torch.empty(batch, rows, dtype=torch.float32, device=w.device)
+    v = torch.empty(batch, cols, dtype=torch.float32, device=w.device)
+    ptrs = (ctypes.c_void_p * batch)(*[mats[b].data_ptr() for b in range(batch)])
+    prob = (_lib.SnProblem * 1)()
+    q = prob[0]
+    q.w_ptrs, q.sigma_out = ctypes.cast(ptrs, ctypes.POINTER(ctypes.c_void_p)), sigma.data_ptr()
+    q.dtype, q.ld, q.batch, q.rows, q.cols = _lib.dtype_code(mats.dtype), mats.stride(-2), batch, rows, cols
+    L = _lib.lib()
+    ws = _lib.workspace(w.device, L.muon_spectral_norm_workspace_bytes(prob, 1), tag="sn")
+    with torch.cuda.device(w.device):
+        st = L.muon_power_iteration(ctypes.cast(ptrs, ctypes.POINTER(ctypes.c_void_p)), q.dtype, q.ld, batch, rows, cols,
+                                    steps, sigma.data_ptr(), u.data_ptr(), v.data_ptr(), ws.data_ptr(), ws.numel(),
+                                    _lib.current_stream_ptr(w.device))
+    _lib.check(st, "muon_power_iteration")
+    lead = w.shape[:-2]
+    u = torch.nn.functional.normalize(u, dim=-1).to(torch.bfloat16).reshape(*lead, rows, 1)
+    v = torch.nn.functional.normalize(v, dim=-1).to(torch.bfloat16).reshape(*lead, cols, 1)
+    return sigma.reshape(lead), u, v
 
 
 @torch.no_grad()

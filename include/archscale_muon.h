@@ -325,6 +325,16 @@ size_t muon_spectral_norm_workspace_bytes(const muon_sn_problem* problems_host, 
 int muon_spectral_norm(const muon_sn_problem* problems_host, int n_problems, int steps, void* workspace_dev,
                        size_t workspace_bytes, void* stream);
 
+/* power_iteration with its singular vectors (spectral_ball_utils.py:151-166 returns (sigma, u, v)): one shape class
+ * as in muon_sn_problem (w_ptrs_host: HOST array of `batch` device pointers; dtype, ld, rows, cols as there), sigma as
+ * muon_spectral_norm computes it, plus the vectors of the same sequence, UNNORMALISED, in fp32:
+ *   u_out_dev [batch][rows]  proportional to W v_steps,   v_out_dev [batch][cols]  proportional to v_steps = (W^T W)^steps 1
+ * (the short-side one is the last Gram-side iterate, the long-side one a single pass over the bf16 copy of W).
+ * Workspace: muon_spectral_norm_workspace_bytes of the same problem. */
+int muon_power_iteration(const void* const* w_ptrs_host, int dtype, int ld, int batch, int rows, int cols, int steps,
+                         float* sigma_out_dev, float* u_out_dev, float* v_out_dev, void* workspace_dev,
+                         size_t workspace_bytes, void* stream);
+
 /* muon_ball_apply: for every item (a strided rows x cols block of a weight tensor)
  *   W <- f * decay * W - lr * lr_ratio * Phi
  * decay = 1 - lr*wd (decoupled) or 1 - wd (independent) or 1 (emerging_optimizers/mixin.py:33-52, applied before the

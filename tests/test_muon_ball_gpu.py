@@ -408,3 +408,39 @@ def test_orthogonalize_per_tensor(gpu_device, case, retract_mode):
         p.add_(upd.to(p.dtype), alpha=-0.02)
     x.add_(want, alpha=-0.02)
     assert _rel(p.detach(), x) <= W_TOL
+
+
+@pytest.mark.parametrize("shape", [(48, 160), (160, 48), (64, 64), (3, 100, 260), (2, 2, 300, 72), (1, 40), (40, 1)])
+@pytest.mark.parametrize("steps", [1, 7, 50])
+def test_power_iteration_vectors(gpu_device, shape, steps):
+    """(sigma, u, v) of the reference's power_iteration (spectral_ball_utils.py:151-166) from the library: against the same
+    vector sequence in fp64, v_k = normalize(W^T W v_{k-1}) from the all-ones vector, u = normalize(W v), sigma = |W v|."""
+    from archscale_amd.emerging.spectral_ball_utils import power_iteration, spectral_norm
+    g = torch.Generator().manual_seed(sum(shape) + steps)
+    W = (torch.randn(*shape, generator=g) * 0.02).to(torch.bfloat16)
+    sigma, u, v = power_iteration(W.to(gpu_device), steps)
+    torch.cuda.synchronize()
+    rows, cols = shape[-2:]
+    assert sigma.shape == shape[:-2] and u.shape == (*shape[:-2], rows, 1) and v.shape == (*shape[:-2], cols, 1)
+    assert u.dtype == torch.bfloat16 and v.dtype == torch.bfloat16
+    assert torch.equal(sigma, spectral_norm(W.to(gpu_device), steps))          # the same sigma as the norm-only entry
+    Wd = W.double().reshape(-1, rows, cols)
+    for b in range(Wd.shape[0]):
+        vv = torch.ones(cols, 1, dtype=torch.float64)
+        for _ in range(steps):
+            vv = Wd[b].T @ (Wd[b] @ vv)
+            vv = vv / vv.norm()
+        uu = Wd[b] @ vv
+        s_ref = uu.norm().item()
+        uu = uu / uu.norm()
+        ub = u.reshape(-1, rows, 1)[b].double().cpu()
+        vb = v.reshape(-1, cols, 1)[b].double().cpu()
+        assert abs(sigma.reshape(-1)[b].item() - s_ref) <= 1e-2 * s_ref      # (sigma itself: the tests above)
+        assert abs(ub.norm().item() - 1) < 1e-2 and abs(vb.norm().item() - 1) < 1e-2
+        # the pair realises the estimate: u^T W v = sigma (second-order in the direction error of either vector)
+        assert (ub.T @ Wd[b] @ vb).item() == pytest.approx(s_ref, rel=1.5e-2)
+        if steps <= 7:
+            # far from convergence the sequence itself is the definition: same direction and sign as in fp64, to the three
+            # digits of a bf16 unit vector (after many rounds the direction inside a cluster of close singular values
+            # depends on the rounding of the Gram matrix, in the reference's bf16 arithmetic as much as here)
+            assert (ub - uu).norm().item() <= 1.5e-2 and (vb - vv).norm().item() <= 1.5e-2, (b, (ub - uu).norm(), (vb - vv).norm())
