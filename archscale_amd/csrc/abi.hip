@@ -72,6 +72,9 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
 }
 
 inline long sym_tiles(int t) { return (long)t * (t + 1) / 2; }
+// matrix-core work of the upper-triangle tiles, in tiles: a diagonal tile runs three quarters of its MFMAs (the waves
+// whose sub-tiles lie wholly below the diagonal sit out)
+inline double sym_tiles_issued(int t) { return (double)sym_tiles(t) - 0.25 * t; }
 
 // workspace bound of one problem: the larger of the two tile configurations (a call with few tiles in total takes the
 // small one, see ns_grouped_impl)
@@ -230,7 +233,7 @@ void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode, doub
   if (symmetric) *symmetric = bi * (3.0 * m * m * n + m * m * m);
   if (issued) {
     const double t = p.tile, tm = p.Mp / p.tile, tn = p.Np / p.tile;
-    const double st = (double)sym_tiles(p.Mp / p.tile);
+    const double st = sym_tiles_issued(p.Mp / p.tile);
     const double passes = prec_mode == MUON_PREC_BF16_BSPLIT ? 2.0 : 1.0;
     *issued = bi * 2.0 * t * t * (st * p.Np + st * p.Mp + tm * tn * p.Mp * passes);
   }
@@ -517,7 +520,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.scale = (P.defer && it == 0) ? P.scale : nullptr;
       const double bm = P.q.batch, dm = pl.m, dn = pl.n, tl = pl.tile;
       fa = bm * dm * dm * dn;
-      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Np;
+      fi = bm * 2.0 * tl * tl * sym_tiles_issued(pl.Mp / pl.tile) * pl.Np;
       return true;
     });
   };
@@ -537,7 +540,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.diag_add = k.fold ? ldexpf(k.a, k.SBi) : 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
-      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
+      fi = bm * 2.0 * tl * tl * sym_tiles_issued(pl.Mp / pl.tile) * pl.Mp;
       return true;
     });
   };
@@ -555,7 +558,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       g.alpha = ldexpf(1.f, shift); g.beta = 0.f;
       const double bm = P.q.batch, dm = pl.m, tl = pl.tile;
       fa = bm * dm * dm * dm;
-      fi = bm * 2.0 * tl * tl * (double)sym_tiles(pl.Mp / pl.tile) * pl.Mp;
+      fi = bm * 2.0 * tl * tl * sym_tiles_issued(pl.Mp / pl.tile) * pl.Mp;
       return true;
     });
   };

@@ -216,6 +216,15 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
 
   const int wr0 = (wave / WAVES_N) * WM;  // wave origin inside the block tile
   const int wc0 = (wave % WAVES_N) * WN;
+  // Diagonal tile of a symmetric product: a wave whose sub-tile lies wholly BELOW the diagonal computes nothing (it
+  // only takes part in the copies and the barriers); its part of the tile is the mirror image of the sub-tiles that
+  // lie wholly ABOVE the diagonal, and those waves write it (two of eight waves idle in the 256x256 configuration, one
+  // of four in the 128x128 one: a quarter of the tile's matrix-core work).
+  static_assert((BM == 256 && BN == 256 && WM == 128 && WN == 64) || (BM == 128 && BN == 128 && WM == 64 && WN == 64),
+                "checked for these two: the idle sub-tiles together are exactly the mirror image of the sub-tiles above the diagonal");
+  const bool diag = SYM && (ti == tj);
+  const bool idle = diag && (wc0 + WN <= wr0);
+  const bool above = diag && (wr0 + WM <= wc0);
   // operand read offsets: row (w0 + i*32 + l32), chunk (2*kk + hi)
   int rdP[4], rdQ[4];
 #pragma unroll
@@ -370,11 +379,27 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
+  if (!idle) {
 #pragma unroll
-  for (int r = 0; r < NRD; ++r) fread(0, smem, smem + PBYTES, 0, r);
-  for (int kt = 0; kt + 2 < KT_ALL; ++kt) ktile(kt, Yes{}, Yes{}, Yes{});
-  if (KT_ALL > 1) ktile(KT_ALL - 2, Yes{}, Yes{}, No{});
-  ktile(KT_ALL - 1, No{}, No{}, No{});
+    for (int r = 0; r < NRD; ++r) fread(0, smem, smem + PBYTES, 0, r);
+    for (int kt = 0; kt + 2 < KT_ALL; ++kt) ktile(kt, Yes{}, Yes{}, Yes{});
+    if (KT_ALL > 1) ktile(KT_ALL - 2, Yes{}, Yes{}, No{});
+    ktile(KT_ALL - 1, No{}, No{}, No{});
+  } else {
+    // an idle wave keeps its share of the copies and meets every barrier of the loop above (one per k-tile that has a
+    // successor), in the same order: rest of k-tile kt+1, barrier, first copies of k-tile kt+2
+    for (int kt = 0; kt + 1 < KT_ALL; ++kt) {
+#pragma unroll
+      for (int g = G1; g < NGL; ++g) gload(kt + 1, g);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      if (kt + 2 < KT_ALL) {
+#pragma unroll
+        for (int g = 0; g < G1; ++g) gload(kt + 2, g);
+      }
+    }
+  }
 
   // ---- epilogue.  acc[i][j][e] of lane l is element
   //   rl = wr0 + i*32 + 8*(e/4) + 4*(l/32) + e%4  (row in the tile),   cl = wc0 + j*32 + l%32  (column)
@@ -397,7 +422,6 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const float sc = p.scale ? p.scale[b] : 1.f;
   const float bx_sc = sc * __builtin_ldexpf(1.f, p.out_shift);   // MODE_BX: scale of the result (a power of two from the host)
   const float alpha = SYRK_PLAIN ? p.alpha * sc * sc : p.alpha, beta = p.beta;
-  const bool diag = SYM && (ti == tj);
   // A diagonal tile of a product of a matrix with ITSELF is symmetric bit for bit as it comes out of the matrix cores
   // (element (i,j) and element (j,i) are the same products summed in the same order over k), so it takes the wave-local
   // epilogue below like any other tile and writes one image.  A diagonal tile of P Q^T with two different (commuting,
@@ -443,6 +467,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   __syncthreads();  // every wave is done reading the operand stages
 
   if (!reflect) {
+    if (idle) return;
     // ---- wave-local epilogue (every tile except the diagonal tiles of a product of two different matrices).
     // Each wave stages its own WM x WN sub-tile in its own LDS region as the transposed image
     // W[c][r] (c = column in the sub-tile, r = row), so nothing below needs a block barrier:
@@ -548,7 +573,7 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
                 pk4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
       // transposed / mirrored image: rows of W
       __bf16* Tdst = SYM ? Cdst : p.Ct;
-      if (Tdst && !diag) {   // a diagonal tile is its own mirror image
+      if (Tdst && (!diag || above)) {   // in a diagonal tile: only the image of the idle waves' part
         const long tbs = SYM ? p.strideC : p.strideCt;
         const int tld = SYM ? p.ldc : p.ldct;
         __bf16* base = Tdst + (size_t)b * tbs;

@@ -150,7 +150,8 @@ void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
  *   key               tile*100 + mode*10 + 4*noaddend + split*2 + final  (mode 0 = X X^T, 1 = cAA+bA, 2 = aX + BX,
  *                     3 = X X^T from the transposed iterate; noaddend: an X' = (B + aI) X launch)
  *   flops_algorithmic minimum FLOPs of the product (symmetric products counted once)
- *   flops_issued      FLOPs of the tiles actually launched
+ *   flops_issued      FLOPs of the matrix-core instructions actually issued (whole tiles; three quarters of a diagonal
+ *                     tile of a symmetric product)
  */
 int muon_profile_begin(void);
 int muon_profile_collect(float* ms_host, int32_t* key_host, double* flops_algorithmic_host,

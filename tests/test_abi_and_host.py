@@ -215,9 +215,10 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
 
     # template arguments of an instantiation from its mangled name: <BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>
     targs = re.compile(r"ns_gemm_kernelILi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])ELb([01])ELi(\d+)EE")
-    seen, reads_of = set(), {}
+    # pass 1: cut every K-major instantiation into basic blocks (label -> instructions, each tagged "inline asm or not")
+    seen, reads_of, kernels = set(), {}, {}
     all_kernels = 0
-    pending, inside, in_asm, cur = set(), False, False, None
+    inside, in_asm, cur, blocks, label = False, False, None, None, None
     for line in text:
         if "#ASMSTART" in line or "#ASMEND" in line:
             in_asm = "#ASMSTART" in line
@@ -234,25 +235,72 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
                 assert cur not in seen, f"{code} seen twice"
                 seen.add(cur)
                 reads_of[cur] = 0
-            pending = set()
+                label = "<entry>"
+                blocks = kernels[cur] = [[label, []]]
             continue
-        if not inside or not code or code.startswith("."):
+        if not inside or not code:
             continue
-        if code.startswith("s_endpgm"):
-            assert not pending
+        if code.startswith(".Lfunc_end"):   # (blocks may follow the first s_endpgm: the function ends here)
             inside = False
             continue
-        if code.startswith("ds_read_b64_tr_b16") and in_asm:   # the compiler tracks the ones it emits itself
-            dst, addr = code[len("ds_read_b64_tr_b16"):].split(",")[:2]
-            assert not (regs(addr) & pending), line
-            assert not (regs(dst) & pending), line
-            pending |= regs(dst)
-            reads_of[cur] += 1
+        if code.endswith(":") and code.startswith(".LBB"):
+            label = code[:-1]
+            blocks.append([label, []])
             continue
-        if code.startswith("s_waitcnt") and "lgkmcnt(0)" in code:
-            pending = set()
+        if code.startswith("."):
             continue
-        assert not (regs(code) & pending), f"uses a transpose-read result before the wait: {line}"
+        blocks[-1][1].append((code, in_asm))
+        if code.startswith(("s_cbranch", "s_branch", "s_endpgm")):
+            blocks.append([f"<after {len(blocks)}>", []])   # a branch or the end of the program ends its block
+
+    # pass 2, per kernel: the set of registers with a transpose read in flight at the entry of each block is the union
+    # over its predecessors (fall-through, conditional and unconditional branches, loop back-edges included), iterated
+    # to a fixed point; then no instruction may mention a register that is pending where it stands
+    def walk(instrs, pending, check, key):
+        pending = set(pending)
+        for code, asm in instrs:
+            if code.startswith("ds_read_b64_tr_b16") and asm:   # the compiler tracks the ones it emits itself
+                dst, addr = code[len("ds_read_b64_tr_b16"):].split(",")[:2]
+                if check:
+                    assert not (regs(addr) & pending), code
+                    assert not (regs(dst) & pending), code
+                    reads_of[key] += 1
+                pending |= regs(dst)
+            elif code.startswith("s_waitcnt") and "lgkmcnt(0)" in code:
+                pending = set()
+            elif check:
+                assert not (regs(code) & pending), f"uses a transpose-read result before the wait: {code}"
+        return pending
+
+    for key, blocks in kernels.items():
+        index = {lab: i for i, (lab, _) in enumerate(blocks)}
+        succ = []
+        for i, (lab, instrs) in enumerate(blocks):
+            out = set()
+            last = instrs[-1][0] if instrs else ""
+            assert not any(c.startswith(("s_cbranch", "s_branch", "s_setpc", "s_swappc")) for c, _ in instrs[:-1]), lab
+            assert not last.startswith(("s_setpc", "s_swappc")), f"indirect jump in {key}"
+            if last.startswith(("s_cbranch", "s_branch")):
+                target = last.split()[-1]
+                assert target in index, f"branch to an unknown label: {last}"
+                out.add(index[target])
+            if not (last.startswith("s_branch") or last.startswith("s_endpgm")) and i + 1 < len(blocks):
+                out.add(i + 1)
+            succ.append(out)
+        pend_in = [set() for _ in blocks]
+        changed = True
+        while changed:
+            changed = False
+            for i, (lab, instrs) in enumerate(blocks):
+                out = walk(instrs, pend_in[i], False, key)
+                for j in succ[i]:
+                    if not out <= pend_in[j]:
+                        pend_in[j] |= out
+                        changed = True
+        for i, (lab, instrs) in enumerate(blocks):
+            out = walk(instrs, pend_in[i], True, key)
+            if instrs and instrs[-1][0].startswith("s_endpgm"):
+                assert not out, f"{key}: transpose reads in flight at the end of the program"
     # every K-major instantiation was visited by name: two tile configurations x {bfloat16, half} workspace
     assert seen == {(256, 0), (256, 1), (128, 0), (128, 1)}, seen
     assert all_kernels > len(seen)
