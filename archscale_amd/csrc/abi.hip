@@ -328,7 +328,9 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     P.partial = (float*)(ws + P.pl.off_partial);
     P.scale = (float*)(ws + P.pl.off_scale);
     P.pow2 = P.scale + P.q.batch;
-    P.tall = P.q.rows > P.q.cols;
+    // a square matrix counts as tall: orthogonalising X^T and transposing the result is the same map, and a tall
+    // matrix enters the workspace as it is (a linear pass instead of a tile transpose)
+    P.tall = P.q.rows >= P.q.cols;
     // An input that is bfloat16 already (or is rounded to it before its norm) goes into the workspace EXACTLY and the
     // factor is applied by the first iteration's epilogues, as after the fused momentum (all but a power of two, which
     // the copy takes exactly and which keeps the products of the first iteration in range): rounding the normalised copy a

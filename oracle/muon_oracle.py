@@ -155,6 +155,8 @@ def newton_schulz(
     if G.ndim < 2:
         raise ValueError("Newton-Schulz needs at least 2 dimensions")
     tall = G.size(-2) > G.size(-1)
+    if storage in ("bf16_gemm", "f16_gemm") and G.size(-2) == G.size(-1):
+        tall = True   # the models of the HIP path follow its orientation: it iterates on the transpose of a square matrix
     X = G.to(torch.bfloat16)
     if tall:
         X = X.mT
