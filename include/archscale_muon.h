@@ -89,7 +89,8 @@ const char* muon_status_string(int status);
  * abc : HOST array of 3*iters floats, one (a, b, c) row per iteration (the reference has three different
  *       tables; none is compiled in).
  * Each matrix is normalised by its own Frobenius norm, tall matrices (rows > cols) are iterated transposed
- * and returned in the caller's orientation.  A bf16 input (or an fp32 one with MUON_NS_CAST_INPUT_FIRST) is not rounded
+ * and returned in the caller's orientation (a square matrix too: orthogonalising the transpose and transposing the
+ * result is the same map, and its memory image is then the operand of the iteration as it is).  A bf16 input (or an fp32 one with MUON_NS_CAST_INPUT_FIRST) is not rounded
  * a second time after the normalisation: the workspace takes it times a power of two, exactly, and the rest of the
  * factor is applied in fp32 by the products of the first iteration.
  * ws  : device workspace of at least muon_ns_workspace_bytes(...) bytes, 256-byte aligned.
