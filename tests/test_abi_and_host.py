@@ -140,6 +140,47 @@ def test_constructor_validation_and_defaults():
         Muon([v]).step()
 
 
+def test_loads_a_state_dict_in_the_reference_layout():
+    """A checkpoint written by the reference's optimizer (torch.optim.Optimizer.state_dict() of lit_gpt/optim/muon.py:86-101,
+    199-209: param-group keys lr, mu, beta1, beta2, weight_decay, cautious_wd, algorithm, step, epsilon, nesterov, flatten,
+    adjust_lr plus the trainer's lr_mult; per-parameter state "momentum", and "variance" in the adamw groups) loads into
+    the drop-in, which then goes on counting steps from the loaded value and hands the same dictionary back."""
+    from archscale_amd.optim.muon import Muon
+    w = torch.nn.Parameter(torch.randn(8, 16))
+    e = torch.nn.Parameter(torch.randn(32, 8))
+    b = torch.nn.Parameter(torch.randn(8))
+    common = dict(mu=0.95, beta1=0.9, beta2=0.95, cautious_wd=False, epsilon=1e-8, nesterov=True, flatten=False,
+                  adjust_lr="spectral_norm")
+    ref_sd = {
+        "state": {
+            0: {"momentum": torch.full((8, 16), 0.25)},
+            1: {"momentum": torch.full((32, 8), -0.5), "variance": torch.full((32, 8), 2.0)},
+            2: {"momentum": torch.full((8,), 0.125), "variance": torch.full((8,), 3.0)},
+        },
+        "param_groups": [
+            dict(common, lr=0.02, weight_decay=0.0, algorithm="muon", step=1234, lr_mult=1.0, params=[0]),
+            dict(common, lr=0.004, weight_decay=0.1, algorithm="adamw", step=1234, lr_mult=0.2, params=[1, 2]),
+        ],
+    }
+    opt = Muon([dict(params=[w]), dict(params=[e, b], algorithm="adamw", lr=0.1)], lr=0.5, use_muonh=True)
+    opt.load_state_dict(ref_sd)
+    g0, g1 = opt.param_groups
+    assert g0["step"] == 1234 and g0["lr"] == 0.02 and g0["algorithm"] == "muon" and g0["lr_mult"] == 1.0
+    assert g1["step"] == 1234 and g1["lr"] == 0.004 and g1["algorithm"] == "adamw" and g1["weight_decay"] == 0.1
+    assert torch.equal(opt.state[w]["momentum"], torch.full((8, 16), 0.25))
+    assert torch.equal(opt.state[e]["variance"], torch.full((32, 8), 2.0))
+    assert torch.equal(opt.state[b]["momentum"], torch.full((8,), 0.125))
+    back = opt.state_dict()
+    assert [sorted(g.keys()) for g in back["param_groups"]] == [sorted(g.keys()) for g in ref_sd["param_groups"]]
+    assert sorted(back["state"][1].keys()) == ["momentum", "variance"] and sorted(back["state"][0].keys()) == ["momentum"]
+    # the step counter continues from the loaded value (counted before the work, which needs the GPU)
+    from archscale_amd._lib import MuonLibraryError
+    w.grad = torch.randn(8, 16)
+    with pytest.raises(MuonLibraryError):
+        opt.step()
+    assert opt.param_groups[0]["step"] == 1235 and opt.param_groups[1]["step"] == 1235
+
+
 def test_lr_ratios_flatten_policy_and_batches():
     from archscale_amd.optim import muon as M
     from archscale_amd.optim.opt_utils import create_param_batches, matrix_view_shape
