@@ -150,6 +150,35 @@ def test_config5_moe_full_step(gpu_device):
         assert _rel(got, x2) < 0.3 * _rel(w0[(i, e)], x2)
 
 
+@pytest.mark.parametrize("config,shapes", [
+    ("config 2", [(512, 2048), (2048, 2048), (2048, 5632), (5632, 2048)]),
+    ("config 5", [(768, 3072), (3072, 1536), (3, 768, 3072), (3, 3072, 384)]),
+])
+def test_singular_values_land_in_the_band(gpu_device, config, shapes):
+    """One matrix of every shape class of the depth-16 and depth-24 parameter sets through ONE grouped Newton-Schulz call
+    (the launch pattern of the optimizer step, classes of different tile counts and K in the same launches): each result
+    within 1e-2 of the fp32 oracle, and its singular values inside the band that the scalar map of the production
+    table assigns to the input's normalised spectrum (lit_gpt/optim/muon.py:875-897)."""
+    import archscale_amd.optim.newton_schulz_hip as H
+    g = torch.Generator().manual_seed(1243)
+    ins = [(torch.randn(*s, generator=g) * 1e-3).to(torch.bfloat16) for s in shapes]
+    outs = H.newton_schulz_grouped([x.to(gpu_device) for x in ins], O.QUINTIC, 1e-7)
+    torch.cuda.synchronize()
+    for x, o in zip(ins, outs):
+        mats_in = x if x.ndim == 3 else x[None]
+        mats_out = (o if o.ndim == 3 else o[None]).cpu()
+        for gi, go in zip(mats_in, mats_out):
+            want = O.newton_schulz(gi, O.QUINTIC, 1e-7, storage="fp32")
+            err = _rel(go, want)
+            s_in = torch.linalg.svdvals(gi.double()) / gi.double().norm()
+            band = O.ns_singular_value_map(s_in, O.QUINTIC)
+            s_out = torch.linalg.svdvals(go.double())
+            print(config, tuple(gi.shape), "err", err, "sv", s_out.min().item(), s_out.max().item(), "band",
+                  band.min().item(), band.max().item(), flush=True)
+            assert err <= NS_TOL
+            assert s_out.min().item() >= band.min().item() - 0.02 and s_out.max().item() <= band.max().item() + 0.02
+
+
 def test_config2_muon_ball_full_step(gpu_device):
     """MuonBall over the depth-16 dense parameter set (112 matrices): 50 power-iteration rounds, hard retraction,
     msign with the polar-express table. Sampled matrices against the CPU oracle, every matrix against the sphere."""

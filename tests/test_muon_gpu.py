@@ -260,31 +260,70 @@ def test_emerging_hook_path(gpu_device):
     assert opt.get_grad_rms_dict()["blk.w"] == pytest.approx((0.1 * g).pow(2).mean().sqrt().item(), rel=1e-3)
 
 
+def _sv_in_band(out, G, coeffs, tol=0.02):
+    """Singular values of an orthogonalised matrix against the band that the scalar map of the coefficient table
+    assigns to the normalised singular values of its input (lit_gpt/optim/muon.py:875-897 in exact arithmetic)."""
+    s_in = torch.linalg.svdvals(G.double().cpu()) / G.double().cpu().norm()
+    band = O.ns_singular_value_map(s_in, coeffs)
+    s_out = torch.linalg.svdvals(out.double().cpu())
+    return s_out.min().item() >= band.min().item() - tol and s_out.max().item() <= band.max().item() + tol
+
+
 def test_config3_expert_batches(gpu_device):
-    """64 experts, W1/W3 stacked 512x2048 and W2 2048x256 (tall => transposed), one batched launch per
-    kernel, per-expert MuonH renormalisation; checked on a seeded subset of experts against the oracle."""
+    """64 experts, W1/W3 stacked 512x2048 and W2 2048x256 (tall => transposed), one batched launch per kernel, per-expert
+    MuonH renormalisation (lit_gpt/optim/muon.py:309-322, 754-758 applied per expert).
+    (i) the 64-batch 3-D Newton-Schulz call of either stack against the fp32 oracle on nine experts each, with the
+        singular values in the band of the table;
+    (ii) the full MuonH step with bf16 weights (the benchmark's configuration): weights within 2e-2 of the
+        reference-semantics oracle (bf16 eager) and of the fp32-NS oracle, norms kept per expert;
+    (iii) the same step with fp32 weights, where the weight DELTA is meaningful: within 3e-2 of the fp32-NS oracle."""
     from archscale_amd.optim.muon import Muon
+    import archscale_amd.optim.newton_schulz_hip as H
     shapes = [(64, 512, 2048), (64, 2048, 256)]
     g = torch.Generator().manual_seed(1237)
     W = [(torch.randn(*s, generator=g) * 0.02).to(torch.bfloat16) for s in shapes]
     G = [(torch.randn(*s, generator=g) * 1e-3).to(torch.bfloat16) for s in shapes]
-    params = [torch.nn.Parameter(w.to(gpu_device)) for w in W]
-    opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.0, use_muonh=True, muonh_per_matrix=True)
-    for p, gr in zip(params, G):
-        p.grad = gr.to(gpu_device)
-    opt.step()
-    torch.cuda.synchronize()
-    for p, w, gr in zip(params, W, G):
-        for e in (0, 17, 63):
-            x = w[e].clone()
-            m = torch.zeros_like(x)
-            O.lit_gpt_muon_step(x, gr[e], m, lr=0.02, mu=0.95, wd=0.0, eps=1e-8, nesterov=True,
-                                adjust="spectral_norm", flatten=False, cautious=False, use_muonh=True,
-                                ns_storage="bf16_eager")
-            assert _rel(p[e].detach(), x) <= W_TOL
-            # the update is really there: distance to the OLD weights is ~lr, to the new ones much less
-            assert _rel(p[e].detach(), x) < 0.25 * _rel(w[e], x)
-            assert p[e].float().norm().item() == pytest.approx(w[e].float().norm().item(), rel=2e-3)
+    experts = (0, 1, 9, 17, 26, 31, 40, 55, 63)
+    # (i) at the first step the update that enters Newton-Schulz is the gradient times (1 + mu) (Nesterov, zero
+    # momentum): the batched call on the gradients is the product's own NS input up to that factor
+    for gr in G:
+        got = H.newton_schulz(gr.to(gpu_device), O.QUINTIC, 1e-7)
+        torch.cuda.synchronize()
+        assert got.shape == gr.shape
+        for e in experts:
+            want = O.newton_schulz(gr[e], O.QUINTIC, 1e-7, storage="fp32")
+            assert _rel(got[e], want) <= 1e-2, (tuple(gr.shape), e)
+        for e in experts[:3]:
+            assert _sv_in_band(got[e], gr[e], O.QUINTIC)
+    for wdtype in (torch.bfloat16, torch.float32):
+        params = [torch.nn.Parameter(w.to(wdtype).to(gpu_device)) for w in W]
+        opt = Muon(params, lr=0.02, mu=0.95, nesterov=True, weight_decay=0.0, use_muonh=True, muonh_per_matrix=True)
+        for p, gr in zip(params, G):
+            p.grad = gr.to(wdtype).to(gpu_device)
+        opt.step()
+        torch.cuda.synchronize()
+        for p, w, gr in zip(params, W, G):
+            n_new = p.detach().float().flatten(1).norm(dim=1).cpu()
+            n_old = w.float().flatten(1).norm(dim=1)
+            assert ((n_new / n_old - 1).abs().max().item() < (2e-3 if wdtype == torch.bfloat16 else 1e-4))
+            for e in experts:
+                w0 = w[e].to(wdtype)
+                xf = w0.clone()
+                O.lit_gpt_muon_step(xf, gr[e].to(wdtype), torch.zeros_like(xf), lr=0.02, mu=0.95, wd=0.0, eps=1e-8,
+                                    nesterov=True, adjust="spectral_norm", flatten=False, cautious=False,
+                                    use_muonh=True, ns_storage="fp32")
+                assert _rel(p[e].detach(), xf) <= W_TOL
+                if wdtype == torch.float32:
+                    assert _rel(p[e].detach().cpu() - w0, xf - w0) <= DW_TOL, (tuple(w.shape), e)
+                elif e in experts[:3]:
+                    xr = w0.clone()
+                    O.lit_gpt_muon_step(xr, gr[e], torch.zeros_like(xr), lr=0.02, mu=0.95, wd=0.0, eps=1e-8,
+                                        nesterov=True, adjust="spectral_norm", flatten=False, cautious=False,
+                                        use_muonh=True, ns_storage="bf16_eager")
+                    assert _rel(p[e].detach(), xr) <= W_TOL
+                    # the update is really there: distance to the OLD weights is ~lr, to the new ones much less
+                    assert _rel(p[e].detach(), xr) < 0.25 * _rel(w[e], xr)
+        del opt, params
 
 
 def test_step_replays_under_a_hip_graph(gpu_device):

@@ -318,7 +318,9 @@ def test_random_shapes_strides_and_modes(ns, gpu_device):
     grouped results identical to single calls."""
     import random
     rng = random.Random(20251)
-    tables = {"quintic": ("bf16", 0), "simple": ("bsplit", 3), "msign": ("f16", 0)}
+    # the constant and polar-express tables run in the half-precision workspace, which is what the package itself uses for
+    # them; "simple_bsplit" keeps the bf16 hi+lo pair (a diagnostic mode) in the sweep for its code paths
+    tables = {"quintic": ("bf16", 0), "simple": ("f16", 0), "msign": ("f16", 0), "simple_bsplit": ("bsplit", 3)}
     singles = []
     for case in range(14):
         rows, cols = rng.choice([1, 3, 17, 64, 100, 129, 255, 300, 513]), rng.choice([2, 31, 64, 96, 200, 257, 640, 1025])
@@ -334,7 +336,7 @@ def test_random_shapes_strides_and_modes(ns, gpu_device):
         g = torch.Generator().manual_seed(1000 + case)
         full = torch.randn(batch, rows, cols + pad, generator=g).to(dtype)
         G = full[..., :cols]
-        coeffs = O.coefficient_schedule(table, 5)
+        coeffs = O.coefficient_schedule("simple" if table == "simple_bsplit" else table, 5)
         em = "clamp" if table == "msign" else "add"
         got = ns.newton_schulz(G.to(gpu_device) if pad == 0 else full.to(gpu_device)[..., :cols], coeffs, 1e-7, eps_mode=em,
                                prec=prec, bsplit_tail=tail, diag_fold=fold)
@@ -342,15 +344,16 @@ def test_random_shapes_strides_and_modes(ns, gpu_device):
         assert got.shape == G.shape and torch.isfinite(got.float()).all()
         for b in range(batch):
             want = O.newton_schulz(G[b].to(torch.bfloat16), coeffs, 1e-7, storage="fp32", eps_mode=em)
-            # the bar is stated for the benchmark's shapes; on small matrices the constant and polar-express tables sit
-            # above it with any bf16 storage
-            # (emulated 64x64: 8.5e-3 and 1.4e-2 with the addend in every iteration), and a matrix with a handful of
-            # singular values has no averaging at all (emulated 3x64: up to 2.6e-2 and 3.9e-2)
+            # the contract's 1e-2 from 16 rows up; a matrix with a handful of singular values has no averaging at all
+            # (emulated 3x64 with the polar-express table: 2.2e-2 in half storage, 3.9e-2 in bf16), so below that the bar is
+            # 3e-2.  The hi+lo pair
+            # in bf16 storage holds 1e-2 only from 256 rows up (emulated 64x64: 8.5e-3 .. 1.4e-2) and is not what the
+            # package runs anywhere: below that it is checked for its code paths only, against a loose ceiling.
             small = min(rows, cols)
-            if table == "quintic" or prec == "f16":
-                bar = NS_TOL if small >= 16 else 2 * NS_TOL
-            else:
+            if prec == "bsplit":
                 bar = NS_TOL if small >= 256 else 2 * NS_TOL if small >= 64 else 0.15
+            else:
+                bar = NS_TOL if small >= 16 else 3 * NS_TOL
             assert _rel(got[b], want) <= bar, (case, b)
         if table == "quintic" and dtype == torch.bfloat16 and fold:
             singles.append((G.contiguous().to(gpu_device), got))
