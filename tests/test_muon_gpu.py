@@ -322,7 +322,7 @@ def test_config3_expert_batches(gpu_device):
                                         use_muonh=True, ns_storage="bf16_eager")
                     assert _rel(p[e].detach(), xr) <= W_TOL
                     # the update is really there: distance to the OLD weights is ~lr, to the new ones much less
-                    assert _rel(p[e].detach(), xr) < 0.25 * _rel(w[e], xr)
+                    assert _rel(p[e].detach(), xr) < 0.3 * _rel(w[e], xr)
         del opt, params
 
 
