@@ -30,12 +30,26 @@ struct NsPlan {
   size_t off_xt[2], off_a, off_bh, off_bl, off_partial, off_scale, total;
 };
 
-int pick_tile(int m, int n) {
-  const char* env = getenv("ARCHSCALE_MUON_TILE");
-  if (env) {
-    const int t = atoi(env);
-    if (t == 128 || t == 256) return t;
+// The ARCHSCALE_MUON_* environment is read ONCE, when the first call needs it (debugging switches: a tile configuration
+// forced for every problem, the quartered last round switched off); later changes of the environment are not seen.
+struct EnvSwitches {
+  int tile;       // 0, 128 or 256
+  bool quarter;
+  EnvSwitches() : tile(0), quarter(true) {
+    if (const char* t = getenv("ARCHSCALE_MUON_TILE")) {
+      const int v = atoi(t);
+      if (v == 128 || v == 256) tile = v;
+    }
+    if (const char* q = getenv("ARCHSCALE_MUON_QUARTER")) quarter = atoi(q) != 0;
   }
+};
+const EnvSwitches& env_switches() {
+  static const EnvSwitches e;
+  return e;
+}
+
+int pick_tile(int m, int n) {
+  if (env_switches().tile) return env_switches().tile;
   // padded work, with the small tile charged for its lower arithmetic intensity
   auto cost = [&](int t, double penalty) {
     const double Mp = (double)round_up(m, t), Np = (double)round_up(n, t);
@@ -79,7 +93,7 @@ inline double sym_tiles_issued(int t) { return (double)sym_tiles(t) - 0.25 * t; 
 // workspace bound of one problem: the larger of the two tile configurations (a call with few tiles in total takes the
 // small one, see ns_grouped_impl)
 size_t plan_bytes_bound(int batch, int rows, int cols, int prec_mode) {
-  if (getenv("ARCHSCALE_MUON_TILE")) return make_plan(batch, rows, cols, prec_mode).total;
+  if (env_switches().tile) return make_plan(batch, rows, cols, prec_mode).total;
   return std::max(make_plan(batch, rows, cols, prec_mode, 256).total, make_plan(batch, rows, cols, prec_mode, 128).total);
 }
 
@@ -145,7 +159,7 @@ hipError_t timed_gemm(int tile, int mode, bool split, bool final_, const Grouped
 constexpr int QUARTER_MAX_TAIL = 128, QUARTER_MAX_ALONE = 176;
 hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp, hipStream_t stream,
                          double fa, double fi, int f16) {
-  static const bool enabled = !(getenv("ARCHSCALE_MUON_QUARTER") && atoi(getenv("ARCHSCALE_MUON_QUARTER")) == 0);
+  const bool enabled = env_switches().quarter;
   const int total = gp.tile_start[gp.n_groups];
   const int round = 256;
   const int full = total / round * round, tail = total - full;
@@ -309,7 +323,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     const NsPlan pl = make_plan(q.batch, q.rows, q.cols, prec_mode);
     sym_blocks += (long)q.batch * sym_tiles(pl.Mp / pl.tile);
   }
-  const int force_tile = (!getenv("ARCHSCALE_MUON_TILE") && sym_blocks * 2 < compute_units()) ? 128 : 0;
+  const int force_tile = (!env_switches().tile && sym_blocks * 2 < compute_units()) ? 128 : 0;
   for (int i = 0; i < n_problems; ++i) {
     NsProblem& P = pr[i];
     P.q = problems_host[i];
@@ -867,13 +881,18 @@ int spectral_norm_impl(const muon_sn_problem* problems_host, int n_problems, int
     const NsPlan& pl = P.sp.pl;
     const long xs = (long)pl.Mp * pl.Np;
     const size_t xt = (size_t)(pl.Mp / 64) * (pl.Np / 64);
-    for (int b = 0; b < P.q.batch; ++b) {
+    // one launch per LAYOUT_PTRS_MAX matrices of the class (the matrices are separate allocations: pointers by value)
+    for (int b0 = 0; b0 < P.q.batch; b0 += LAYOUT_PTRS_MAX) {
+      LayoutPtrs lp = {};
+      const int nb = std::min(LAYOUT_PTRS_MAX, P.q.batch - b0);
+      for (int k = 0; k < nb; ++k) lp.p[k] = P.q.w_ptrs[b0 + k];
+      __bf16* dst = P.X + (size_t)b0 * xs;
       if (!P.use_t)
-        e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, P.X + b * xs, xs,
-                          pl.Np, pl.Mp, pl.Np, nullptr, 0, 0, stream, 0, 0, P.xpart + b * xt);
+        e = launch_layout_ptrs(lp, nb, P.q.dtype, P.q.ld, P.q.rows, P.q.cols, dst, xs, pl.Np, pl.Mp, pl.Np, nullptr, 0, 0,
+                               stream, P.xpart + (size_t)b0 * xt);
       else
-        e = launch_layout(P.q.w_ptrs[b], P.q.dtype, 0, 0, P.q.ld, 1, P.q.rows, P.q.cols, nullptr, nullptr, 0, 0,
-                          pl.Np, pl.Mp, P.X + b * xs, xs, pl.Np, stream, 0, 0, P.xpart + b * xt);
+        e = launch_layout_ptrs(lp, nb, P.q.dtype, P.q.ld, P.q.rows, P.q.cols, nullptr, 0, 0, pl.Np, pl.Mp, dst, xs, pl.Np,
+                               stream, P.xpart + (size_t)b0 * xt);
       if (e != hipSuccess) return (int)e;
     }
   }

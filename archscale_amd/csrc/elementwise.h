@@ -41,6 +41,17 @@ hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_b
                          void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16 = 0, int out_shift = 0,
                          float* tile_sumsq = nullptr);
 
+// the same pass over up to LAYOUT_PTRS_MAX matrices of one shape that are separate allocations (pointers by value, as
+// they are: no scale, bf16 output), one launch: matrix i goes to D + i * d_bstride / T + i * t_bstride and its tile sums
+// to tile_sumsq + i * (d_rows / 64) * (d_cols / 64)
+constexpr int LAYOUT_PTRS_MAX = 64;
+struct LayoutPtrs {
+  const void* p[LAYOUT_PTRS_MAX];
+};
+hipError_t launch_layout_ptrs(const LayoutPtrs& ptrs, int n_mats, int in_dtype, int ld, int rows, int cols, void* D,
+                              long d_bstride, int ldd, int d_rows, int d_cols, void* T, long t_bstride, int ldt,
+                              hipStream_t stream, float* tile_sumsq);
+
 // momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
 constexpr int MOMLAY_MAX = 32;
 constexpr int MOMLAY_TILE = 128;   // rows and columns of the tile of one block; one partial sum per tile

@@ -266,7 +266,7 @@ norm_scale_kernel(const float* __restrict__ partial, int chunks_per_mat, float e
 // ---------------------------------------------------------------------------
 template <int DT, bool CAST_FIRST>
 __global__ void __launch_bounds__(256)
-normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, int cols, int ld,
+normalize_layout_kernel(const void* __restrict__ in, const LayoutPtrs ptrs, long in_bstride, int rows, int cols, int ld,
                         const float* __restrict__ scale,
                         uint16_t* __restrict__ D, long d_bstride, int ldd, int d_rows, int d_cols,
                         uint16_t* __restrict__ T, long t_bstride, int ldt, int out_f16, int out_shift,
@@ -277,12 +277,13 @@ normalize_layout_kernel(const void* __restrict__ in, long in_bstride, int rows, 
   float ss[1] = {0.f};
   const int b = blockIdx.z;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-  const char* base = (const char*)in + (size_t)b * in_bstride * sizeof(typename Elem<DT>::T);
+  // the matrices of the batch: equally spaced from `in`, or (in == null) separate allocations listed in `ptrs`
+  const char* base = in ? (const char*)in + (size_t)b * in_bstride * sizeof(typename Elem<DT>::T) : (const char*)ptrs.p[b];
   const float s = scale ? scale[b] : 1.f;
   const float fs = __builtin_ldexpf(1.f, out_shift);
   const int tr = threadIdx.x >> 3;        // 0..31
   const int tc = (threadIdx.x & 7) * 8;   // 0..56
-  const bool vec = aligned16(base) && (ld % 8 == 0) && (in_bstride % 8 == 0);
+  const bool vec = aligned16(base) && (ld % 8 == 0) && (!in || in_bstride % 8 == 0);
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int r = r0 + tr + h * 32, c = c0 + tc;
@@ -351,21 +352,42 @@ hipError_t launch_norm_scale(const void* in, int in_dtype, int cast_first, long 
   return hipGetLastError();
 }
 
-hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
-                         int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
-                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16, int out_shift,
-                         float* tile_sumsq) {
+namespace {
+hipError_t launch_layout_impl(const void* in, const LayoutPtrs& ptrs, int in_dtype, int cast_first, long in_bstride, int ld,
+                              int batch, int rows, int cols, const float* scale, void* D, long d_bstride, int ldd,
+                              int d_rows, int d_cols, void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16,
+                              int out_shift, float* tile_sumsq) {
   if (batch > 65535 || d_rows / 64 > 65535 || d_rows % 64 || d_cols % 64) return hipErrorInvalidValue;
   dim3 g3(d_cols / 64, d_rows / 64, batch);
 #define ARCHSCALE_NL(DT, CF)                                                                                   \
-  hipLaunchKernelGGL((normalize_layout_kernel<DT, CF>), g3, dim3(256), 0, stream, in, in_bstride, rows, cols,  \
-                     ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride, ldt,    \
-                     out_f16, out_shift, tile_sumsq)
+  hipLaunchKernelGGL((normalize_layout_kernel<DT, CF>), g3, dim3(256), 0, stream, in, ptrs, in_bstride, rows,  \
+                     cols, ld, scale, (uint16_t*)D, d_bstride, ldd, d_rows, d_cols, (uint16_t*)T, t_bstride,   \
+                     ldt, out_f16, out_shift, tile_sumsq)
   if (in_dtype == DT_BF16) ARCHSCALE_NL(DT_BF16, false);
   else if (cast_first) ARCHSCALE_NL(DT_F32, true);
   else ARCHSCALE_NL(DT_F32, false);
 #undef ARCHSCALE_NL
   return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_layout(const void* in, int in_dtype, int cast_first, long in_bstride, int ld, int batch, int rows,
+                         int cols, const float* scale, void* D, long d_bstride, int ldd, int d_rows, int d_cols,
+                         void* T, long t_bstride, int ldt, hipStream_t stream, int out_f16, int out_shift,
+                         float* tile_sumsq) {
+  if (!in) return hipErrorInvalidValue;
+  return launch_layout_impl(in, LayoutPtrs{}, in_dtype, cast_first, in_bstride, ld, batch, rows, cols, scale, D, d_bstride,
+                            ldd, d_rows, d_cols, T, t_bstride, ldt, stream, out_f16, out_shift, tile_sumsq);
+}
+
+hipError_t launch_layout_ptrs(const LayoutPtrs& ptrs, int n_mats, int in_dtype, int ld, int rows, int cols, void* D,
+                              long d_bstride, int ldd, int d_rows, int d_cols, void* T, long t_bstride, int ldt,
+                              hipStream_t stream, float* tile_sumsq) {
+  if (n_mats < 1 || n_mats > LAYOUT_PTRS_MAX) return hipErrorInvalidValue;
+  for (int i = 0; i < n_mats; ++i)
+    if (!ptrs.p[i]) return hipErrorInvalidValue;
+  return launch_layout_impl(nullptr, ptrs, in_dtype, 0, 0, ld, n_mats, rows, cols, nullptr, D, d_bstride, ldd, d_rows,
+                            d_cols, T, t_bstride, ldt, stream, 0, 0, tile_sumsq);
 }
 
 // ---------------------------------------------------------------------------

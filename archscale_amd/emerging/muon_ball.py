@@ -478,12 +478,19 @@ class MuonBall(OrthogonalizedOptimizer):
             raise NotImplementedError("MuonBall on MI355X runs on one GPU: tensor-parallel groups must have one rank")
         R = compute_target_radius(tuple(W.shape), self.radius_mode)
         sigma = spectral_norm(W, self.power_iteration_steps)            # 0-d fp32 device tensor
+        # the factor stays in fp32 (the reference multiplies by a Python float in fp32 arithmetic): rounded to bf16 first,
+        # R / sigma would be off by up to 0.4 % and 1 +- alpha * lr would round to exactly 1 for a small lr
+        def scale_(factor: torch.Tensor) -> None:
+            if W.dtype == torch.float32:
+                W.mul_(factor)
+            else:
+                W.copy_(W.to(torch.float32) * factor)
         if self.retract_mode == "hard":
-            W.mul_((R / (sigma.clamp_min(0.0) + 1e-8)).to(W.dtype))
+            scale_(R / (sigma.clamp_min(0.0) + 1e-8))
         else:
             bias_t = torch.where(sigma > R, -1.0, 1.0)
             step = self.retract_alpha * current_lr if current_lr is not None else self.retract_alpha
-            W.mul_((1.0 + step * bias_t).to(W.dtype))
+            scale_(1.0 + step * bias_t)
             if param_name and component_label:
                 self.retract_bias_dict[f"{param_name}.{component_label}"] = float(bias_t.item())
                 self.spectral_norm_dict[f"{param_name}.{component_label}"] = float(sigma.item())

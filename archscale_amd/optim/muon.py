@@ -236,8 +236,10 @@ class Muon(Optimizer):
 
     Extra keyword-only knobs of this implementation:
       ns_coefficients   (a, b, c) rows, one per iteration (default: the reference's 5-row schedule)
-      ns_precision      "bf16", "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair) or "f16" (the iteration's matrices
-                        in IEEE half inside the workspace, scaled by powers of two: 8x the mantissa at the same rate)
+      ns_precision      "bf16" or "f16" (the iteration's matrices in IEEE half inside the workspace, scaled by powers of
+                        two: 8x the mantissa at the same rate; what the constant and polar-express tables need).
+                        "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair, a second walk over K in BX) is still
+                        accepted as a diagnostic mode: "f16" is both faster and more accurate
       muonh_per_matrix  renormalise each matrix of a 3-D parameter on its own instead of the whole tensor
       fuse_momentum     momentum and Newton-Schulz in one library call that never stores the bf16 update in the
                         parameter's orientation (default; falls back to separate calls with a hook or a tight limit)

@@ -88,7 +88,8 @@ def newton_schulz(
     Returns a new bf16 tensor shaped like ``G`` (``G`` itself is not modified unless ``out is G``).
     ``prec="f16"`` keeps the iterate and both Gram-side matrices in IEEE half inside the workspace (scaled by powers of
     two; 8x the mantissa of bf16 at the same matrix-core rate): what the constant-coefficient and polar-express tables
-    need to stay within 1e-2 of an fp32 run.  ``prec="bsplit"`` stays in bf16 and keeps ``B = bA + cA^2`` as a hi+lo
+    need to stay within 1e-2 of an fp32 run.  ``prec="bsplit"`` is a diagnostic mode that nothing in the package uses
+    (slower and less accurate than "f16"): it stays in bf16 and keeps ``B = bA + cA^2`` as a hi+lo
     pair (a second walk over K in ``BX``); ``bsplit_tail=t`` does so only in the
     last ``t`` iterations (0 = all), whose rounding dominates the error of the result.  ``normalize=False`` iterates on
     the input as it is (``epsilon`` is then unused).  ``diag_fold=False`` keeps ``aX`` as a separate addend in every

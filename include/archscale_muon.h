@@ -33,7 +33,8 @@ extern "C" {
 /* precision of B = bA + cA^2 as an operand of B*X */
 #define MUON_PREC_BF16 0       /* one bf16 rounding per GEMM epilogue (rounding points of newton_schulz_triton.py:374-378);
                                   the last two iterations round to IEEE half instead unless MUON_NS_NO_GRAM_TAIL is set */
-#define MUON_PREC_BF16_BSPLIT 1 /* B kept as a bf16 hi+lo pair, B*X accumulates both (needed for the constant-coefficient table) */
+#define MUON_PREC_BF16_BSPLIT 1 /* DIAGNOSTIC mode, superseded by MUON_PREC_F16 (faster: one walk over K per product; a
+                                  third of the error): B kept as a bf16 hi+lo pair, B*X accumulates both */
 #define MUON_PREC_F16 2         /* the iterate and both Gram-side matrices are kept in IEEE half inside the workspace (inputs
                                    and the result stay bfloat16), each times a power of two that keeps it in the normal
                                    range: eight times the mantissa of bfloat16 at the same matrix-core rate, no hi+lo pair
@@ -137,9 +138,12 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems,
                     const float* abc_host, int iters, float eps, int eps_mode, int prec_mode, int flags,
                     void* ws_dev, size_t ws_bytes, void* stream);
 
-/* Algorithmic work of one call, for roofline accounting: dense-count FLOPs (what a GEMM library executes),
- * symmetric-count FLOPs (upper-triangle SYRK minimum) and FLOPs this library issues (tiles incl. padding,
- * full diagonal tiles and the second pass of the B split). */
+/* Algorithmic work of `iters` PLAIN iterations, for roofline accounting: dense-count FLOPs (what a GEMM library
+ * executes), symmetric-count FLOPs (upper-triangle SYRK minimum) and FLOPs this library issues for them (tiles incl.
+ * padding, three quarters of a diagonal tile, the second pass of the B split).  A call that takes the Gram-side tail
+ * (see the flags above) replaces one B X and one X X^T product of every problem with long side >= 2 x short side by three
+ * m x m symmetric products; that is not counted here - the per-launch records of muon_profile_collect are the
+ * authoritative count of what a call issued. */
 void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
                    double* dense, double* symmetric, double* issued);
 

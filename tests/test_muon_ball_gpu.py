@@ -410,6 +410,32 @@ def test_orthogonalize_per_tensor(gpu_device, case, retract_mode):
     assert _rel(p.detach(), x) <= W_TOL
 
 
+@pytest.mark.parametrize("retract_mode", ["hard", "dynamic"])
+def test_orthogonalize_bf16_weights_keep_the_factor_in_fp32(gpu_device, retract_mode):
+    """bf16 parameters through the per-tensor entry: the retraction factor (R / sigma, or 1 +- alpha * lr) multiplies the
+    weights in fp32 and the product is rounded once, as the reference's ``W.mul_(python_float)`` does
+    (muon_ball.py:301-352); the result is what the same factor gives on the host.  A factor rounded to bf16 first would
+    be off by up to 0.4 %."""
+    from archscale_amd.emerging import MuonBall
+    from archscale_amd.emerging.spectral_ball_utils import spectral_norm, compute_target_radius
+    g = torch.Generator().manual_seed(29)
+    W0 = (torch.randn(96, 80, generator=g) * 0.05).to(torch.bfloat16)
+    M0 = (torch.randn(96, 80, generator=g) * 1e-2).to(torch.bfloat16)
+    lr = 0.2      # dynamic mode: factor 1 +- 0.01, which bf16 would round to 1.0078 / 0.9922
+    p = _named(W0.clone().to(gpu_device), "attn.w")
+    opt = MuonBall([p], lr=lr, momentum_beta=0.9, weight_decay=0.0, power_iteration_steps=8, msign_steps=5,
+                   retract_mode=retract_mode)
+    sigma = spectral_norm(W0.to(gpu_device), 8).item()
+    R = compute_target_radius((96, 80), "spectral_mup")
+    opt.orthogonalize(p, M0.clone().to(gpu_device), lr=lr)
+    torch.cuda.synchronize()
+    factor = R / (sigma + 1e-8) if retract_mode == "hard" else 1.0 + 0.05 * lr * (-1.0 if sigma > R else 1.0)
+    want = (W0.float() * torch.tensor(factor, dtype=torch.float32)).to(torch.bfloat16)
+    got = p.detach().cpu()
+    assert (got.float() - want.float()).abs().max().item() <= 2.0 ** -8 * want.float().abs().max().item()   # one bf16 ulp
+    assert _rel(got, W0.double() * factor) <= 1.8e-3      # bf16 rounding of the product only (rms 2^-9 / sqrt(3))
+
+
 @pytest.mark.parametrize("shape", [(48, 160), (160, 48), (64, 64), (3, 100, 260), (2, 2, 300, 72), (1, 40), (40, 1)])
 @pytest.mark.parametrize("steps", [1, 7, 50])
 def test_power_iteration_vectors(gpu_device, shape, steps):

@@ -210,7 +210,7 @@ def test_single_step_without_normalisation(gpu_device, shape):
     Xd = X.double()
     A = Xd @ Xd.T
     want = a * Xd + (b * A + c * A @ A) @ Xd
-    assert _rel(got, want) <= 4e-3          # one bf16 rounding of A, of B (hi+lo) and of the result
+    assert _rel(got, want) <= 4e-3          # one bf16 rounding of A, of B and of the result
     with pytest.raises(ValueError):
         newton_schulz_step_tsyrk(X.float().to(gpu_device), a, b, c)
 
