@@ -240,6 +240,9 @@ class Muon(Optimizer):
                         two: 8x the mantissa at the same rate; what the constant and polar-express tables need).
                         "bsplit" (B = bA + cA^2 kept as a bf16 hi+lo pair, a second walk over K in BX) is still
                         accepted as a diagnostic mode: "f16" is both faster and more accurate
+      ns_gram_tail      None (default): with "bf16" the last two iterations are stored in IEEE half and, for matrices whose
+                        long side is at least twice the short one, finished on the Gram side (one BX and one XX^T
+                        product less); False: five plain iterations; True: the tail also with "f16"
       muonh_per_matrix  renormalise each matrix of a 3-D parameter on its own instead of the whole tensor
       fuse_momentum     momentum and Newton-Schulz in one library call that never stores the bf16 update in the
                         parameter's orientation (default; falls back to separate calls with a hook or a tight limit)
@@ -272,6 +275,7 @@ class Muon(Optimizer):
         *,
         ns_coefficients: Optional[Sequence[Tuple[float, float, float]]] = None,
         ns_precision: str = "bf16",
+        ns_gram_tail: Optional[bool] = None,
         muonh_per_matrix: bool = False,
         ns_workspace_limit: int = 48 << 30,
         fuse_momentum: bool = True,
@@ -324,6 +328,8 @@ class Muon(Optimizer):
         self._newton_schulz_func = newton_schulz_func
         self._ns_coefficients = tuple(tuple(map(float, r)) for r in (ns_coefficients or ns.QUINTIC_SCHEDULE))
         self._ns_precision = ns_precision
+        self._ns_gram_tail = ns_gram_tail
+        self._ns_tail_flags = 0 if ns_gram_tail is None else (_lib.NS_GRAM_TAIL if ns_gram_tail else _lib.NS_NO_GRAM_TAIL)
         self._muonh_per_matrix = muonh_per_matrix
         self._ns_workspace_limit = int(ns_workspace_limit)
         self._fuse_momentum = bool(fuse_momentum)
@@ -518,7 +524,8 @@ class Muon(Optimizer):
         coeffs = self._ns_coefficients
         with self._timed("momentum+newton_schulz"):
             _lib.check(L.muon_momentum_ns_grouped(plan.fused_probs, n, mu, 1.0, c_um, c_ug, 0.0, _lib.abc_array(coeffs),
-                                                  len(coeffs), eps, _lib.EPS_ADD, pm, _lib.ns_bsplit_tail(ns.BSPLIT_TAIL),
+                                                  len(coeffs), eps, _lib.EPS_ADD, pm,
+                                                  _lib.ns_bsplit_tail(ns.BSPLIT_TAIL) | self._ns_tail_flags,
                                                   ws.data_ptr(), ws.numel(), stream), "muon_momentum_ns_grouped")
         return True
 
@@ -534,7 +541,7 @@ class Muon(Optimizer):
             nonlocal parts, used
             if parts:
                 ns.newton_schulz_grouped(parts, self._ns_coefficients, eps, prec=self._ns_precision, outs=parts,
-                                         bsplit_tail=ns.BSPLIT_TAIL)
+                                         bsplit_tail=ns.BSPLIT_TAIL, gram_tail=self._ns_gram_tail)
             parts, used = [], 0
 
         for cls in classes:

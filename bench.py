@@ -5,9 +5,12 @@ A "step" is one full MuonH optimizer step (momentum -> Newton-Schulz-5 -> hypers
 weight of the depth-16 GQA transformer parameter set: 112 bf16 matrices, 721.4 M elements, seeded synthetic
 weights N(0, 0.02^2) and gradients N(0, 1e-3^2), resident in HBM before the timed region.
 
-Prints ONE JSON line: headline = dense-count Newton-Schulz TFLOP/s over the whole step (what a GEMM library
-would execute: 5*(4 m^2 n + 2 m^3) per matrix), ms per step, the roofline of the dominant kernel measured
-with HIP events per launch, and the CPU baseline (the oracle's eager-bf16 restatement of the reference's CPU
+Prints ONE JSON line: headline = matrix-core FLOPs that the step EXECUTES (the library's own count per GEMM launch:
+whole tiles, upper triangles only, the products of the Gram-side tail as they are) over the wall time of the whole step
+(GEMMs and HBM-bound kernels), so value / 2500 is the share of the bf16 peak that the whole step sustains; beside it the
+dense-equivalent figure (what a GEMM library or the CPU path would execute: 5*(4 m^2 n + 2 m^3) per matrix), ms per
+step, the same step with five plain iterations (no half-storage / Gram-side tail), the roofline of the dominant kernel
+measured with HIP events per launch, and the CPU baseline (the oracle's eager-bf16 restatement of the reference's CPU
 path) timed on a bounded sample in the same run.
 """
 from __future__ import annotations
@@ -129,7 +132,7 @@ def other_configs(dev, which):
     def pack(ms, shapes_counts, recs, **extra):
         dense = sum(c * dense_flops(s) for s, c in shapes_counts)
         gms, fi, fa = _gemm_summary(recs)
-        d = {"ms": round(ms, 4), "dense_tflops": round(dense / ms / 1e9, 1),
+        d = {"ms": round(ms, 4), "executed_tflops": round(fi / ms / 1e9, 1), "dense_equivalent_tflops": round(dense / ms / 1e9, 1),
              "gemm_ms": round(gms, 4),
              "gemm_pct_mfma_peak_issued": round(fi / gms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2) if gms else None,
              "gemm_pct_mfma_peak_algorithmic": round(fa / gms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2) if gms else None}
@@ -188,20 +191,37 @@ def other_configs(dev, which):
 
 
 TRAFFIC_PROFILE = "profiles/bench_config2_ns_gemm_and_epilogues.md"
+GEMM_SOURCE = "archscale_amd/csrc/ns_gemm.hip"
+
+
+def source_fingerprint(rel_path):
+    """First 16 hex digits of the SHA-256 of a source file (what a counter summary records about the kernels it measured)."""
+    import hashlib
+    try:
+        return hashlib.sha256(open(os.path.join(ROOT, rel_path), "rb").read()).hexdigest()[:16]
+    except OSError:
+        return None
 
 
 def measured_traffic(kernel_name):
-    """HBM bytes per launch of `kernel_name` from the committed counter summary (two `rocprofv3 --pmc` runs,
-    FETCH_SIZE and WRITE_SIZE, each scaled by the reading of a plain copy of known size), or None."""
+    """(HBM bytes per launch of `kernel_name`, fingerprint of the GEMM source the summary was measured with) from the
+    committed counter summary (two `rocprofv3 --pmc` runs, FETCH_SIZE and WRITE_SIZE, each scaled by the reading of a
+    plain copy of known size).  The byte count is None when the summary is missing or was measured with another version
+    of the GEMM kernels than the one in the tree (a stale figure is not reported)."""
     path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    traffic, measured_with = None, None
     try:
         for line in open(path):
             line = line.strip()
             if line.startswith("traffic_bytes_per_launch") and kernel_name in line:
-                return float(line.split("=")[1])
+                traffic = float(line.split("=")[1])
+            if line.startswith("measured_with_source_sha256_16") and GEMM_SOURCE in line:
+                measured_with = line.split("=")[1].strip()
     except OSError:
         pass
-    return None
+    if measured_with is None or measured_with != source_fingerprint(GEMM_SOURCE):
+        traffic = None
+    return traffic, measured_with
 
 
 def main():
@@ -217,6 +237,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--separate-momentum", action="store_true",
                     help="(comparison) momentum kernel and Newton-Schulz as separate library calls instead of the fused one")
+    ap.add_argument("--no-plain-row", action="store_true",
+                    help="skip the extra timing of the same step with five plain iterations (no half / Gram-side tail)")
     ap.add_argument("--seed", type=int, default=1236)
     ap.add_argument("--min-timed-seconds", type=float, default=2.0,
                     help="the block of --steps steps is repeated until the timed region is at least this long")
@@ -276,6 +298,21 @@ def main():
     for name, a, b in opt.phase_events:
         phases[name] = phases.get(name, 0.0) + a.elapsed_time(b)
     opt.phase_events = None
+
+    # the same step with five plain iterations (no half-storage tail, no Gram-side finish): the figure that stays
+    # comparable when the tail changes the amount of work
+    plain_row = None
+    if not args.no_plain_row and not simple and args.precision == "bf16":
+        opt2 = Muon(params, lr=0.02, mu=0.95, weight_decay=0.0, epsilon=1e-8, nesterov=True, adjust_lr="spectral_norm",
+                    use_muonh=True, ns_gram_tail=False, fuse_momentum=not args.separate_momentum)
+        ms2 = _time_calls(opt2.step, args.steps, warm=2)
+        gms2, fi2, fa2 = _gemm_summary(_instrumented(opt2.step))
+        plain_row = {"ms_per_step": round(ms2, 3), "ns_gemm_ms": round(gms2, 3),
+                     "issued_tflop_per_step": round(fi2 / 1e12, 3),
+                     "executed_tflops": round(fi2 / ms2 / 1e9, 1),
+                     "ns_gemm_pct_mfma_peak_issued": round(fi2 / gms2 / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
+                     "what": "five plain bf16 iterations (ns_gram_tail=False): 15 GEMM launches, bf16 storage throughout"}
+        del opt2
 
     # one plain copy of known size: `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` readings are scaled by what the same
     # counter reports for this dispatch (calibration_copy_kernel)
@@ -349,10 +386,13 @@ def main():
         "issued_frac": round(dom["fi"] / dom["ms"] / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
     }
     if args.layers == N_LAYERS:
-        roofline["traffic"] = measured_traffic(roofline["kernel"])
+        roofline["traffic"], measured_with = measured_traffic(roofline["kernel"])
         # not measured in this run: counters need rocprofv3 passes of their own
         roofline["traffic_source"] = (f"{TRAFFIC_PROFILE} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
-                                      "scaled by the calibration copy; committed summary, not measured in this run)")
+                                      "scaled by the calibration copy; committed summary, not measured in this run; "
+                                      f"null when it was measured with another version of {GEMM_SOURCE})")
+        roofline["traffic_measured_with_source"] = measured_with
+        roofline["source_in_tree"] = source_fingerprint(GEMM_SOURCE)
     if dom_key[1] == 2:  # B (m^2), X^T read (once more as the addend unless a*I is folded into B), X'^T written: bf16
         reads_x = 1 if dom_key[4] else 2
         per = [(min(s) ** 2 + (reads_x + 1) * min(s) * max(s)) * 2.0 for s in shapes]
@@ -386,7 +426,7 @@ def main():
 
     out = {
         "metric": "Muon NS5 TFLOP/s (% bf16 MFMA peak) + MuonH step ms, d16 param set, 1 GPU",
-        "value": round(f_dense / ms_per_step / 1e9, 1),
+        "value": round(f_issued / ms_per_step / 1e9, 1),
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3),
@@ -397,8 +437,20 @@ def main():
                                f"{len(params)} bf16 matrices, {n_elem / 1e6:.1f} M elements, "
                                f"mu 0.95 nesterov, NS5 {args.coeffs} coefficients, lr 0.02, seed {args.seed}",
                    "coefficients": args.coeffs,
-                   "ns_precision": "f16" if args.precision == "f16" else "bsplit" if simple else "bf16"},
-        "value_definition": "dense-count NS FLOPs (5*(4m^2n+2m^3) per matrix) / wall time of the WHOLE step",
+                   "ns_precision": ("f16" if args.precision == "f16" else "bsplit" if simple else
+                                    "bf16; last two iterations in IEEE half, finished on the Gram side for n >= 2m")},
+        "value_definition": "matrix-core FLOPs the step EXECUTES (the library's count per GEMM launch: whole tiles, upper "
+                            "triangles only, three quarters of a diagonal tile, the Gram-side tail's products as they "
+                            "are) / wall time of the WHOLE step; value / 2500 is the share of the bf16 peak over the step",
+        "pct_mfma_peak_whole_step": round(f_issued / ms_per_step / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
+        "issued_tflop_per_step": round(f_issued / 1e12, 3),
+        "symmetric_tflop_per_step": round(f_sym / 1e12, 3),
+        "dense_tflop_per_step": round(f_dense / 1e12, 3),
+        "dense_equivalent_tflops": round(f_dense / ms_per_step / 1e9, 1),
+        "dense_equivalent_definition": "5*(4m^2n+2m^3) per matrix (what a GEMM library or the CPU path executes for five "
+                                       "plain iterations) / wall time of the whole step: a speed-up yardstick against "
+                                       "such a path, NOT a share of the peak (about 0.66 of these FLOPs are executed)",
+        "plain_iterations": plain_row,
         "ns_gemm_pct_mfma_peak_issued": round(f_issued / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
         "ns_gemm_pct_mfma_peak_symmetric": round(f_sym / gemm_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS * 100, 2),
         "ns_gemm_ms": round(gemm_ms, 3), "ns_phase_ms": round(ns_ms, 3),
