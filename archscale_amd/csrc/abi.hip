@@ -390,40 +390,83 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
                         P.q.cols, sc, P.Xt[0], xs, pl.Mp, pl.Np, pl.Mp, nullptr, 0, 0, stream, to_half, to_half ? P.sx : 0);
     if (e != hipSuccess) return (int)e;
   }
-  // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials
-  for (int i = 0; i < n_problems && fused; ++i) {
-    const NsProblem& P = pr[i];
-    const NsPlan& pl = P.pl;
-    const muon_mns_problem& f = fused[i];
-    const long xs = (long)pl.Mp * pl.Np;
-    const int d_rows = P.tall ? pl.Np : pl.Mp, d_cols = P.tall ? pl.Mp : pl.Np;   // padded extents of the matrix itself
-    // a tall matrix whose extents need no padding goes into the workspace as it is: a linear pass, partials per chunk
-    const bool linear = P.tall && P.q.rows == pl.Np && P.q.cols == pl.Mp;
-    const int tiles = linear ? pl.cpm : (d_rows / MOMLAY_TILE) * (d_cols / MOMLAY_TILE);
-    for (int b0 = 0; b0 < P.q.batch; b0 += MOMLAY_MAX) {
-      MomLayoutParams mp = {};
-      mp.n_mats = std::min(MOMLAY_MAX, P.q.batch - b0);
-      mp.rows = P.q.rows; mp.cols = P.q.cols;
-      mp.g_dtype = f.g_dtype; mp.m_dtype = f.m_dtype; mp.w_dtype = f.w_dtype;
-      mp.transpose = P.tall ? 0 : 1;
-      mp.d_rows = d_rows; mp.d_cols = d_cols; mp.ldd = pl.Mp; mp.d_bstride = xs;
-      mp.dst = (uint16_t*)(P.Xt[0] + (size_t)b0 * xs);
-      mp.partial = P.partial + (size_t)b0 * tiles;
-      mp.c = mc;
-      for (int k = 0; k < mp.n_mats; ++k) {
-        mp.g[k] = f.g_ptrs[b0 + k];
-        mp.m[k] = f.m_ptrs[b0 + k];
-        mp.w[k] = f.w_ptrs ? f.w_ptrs[b0 + k] : nullptr;
+  // fused staging: momentum of every matrix, its bf16 update written unnormalised into X^T, norms from tile partials.
+  // The matrices of ALL problems share launches (up to MOMG_MAX_MATS matrices of MOMG_MAX_CLS classes each): one
+  // sequence of launches for the matrices that take the linear pass, one for those that take the tile pass.
+  if (fused) {
+    std::vector<int> blocks_per_mat(n_problems);
+    for (int pass = 0; pass < 2; ++pass) {   // 0: linear pass, 1: tile pass (transposition and / or padding)
+      MomGroupParams mp = {};
+      double bytes = 0.0;
+      auto flush = [&]() -> hipError_t {
+        if (mp.n_mats == 0) return hipSuccess;
+        const double b = bytes;
+        hipError_t err = timed_launch(PROF_KEY_MOMENTUM_LAYOUT, b, b, stream, [&] { return launch_momentum_group(mp, stream); });
+        mp = MomGroupParams{};
+        bytes = 0.0;
+        return err;
+      };
+      for (int i = 0; i < n_problems; ++i) {
+        const NsProblem& P = pr[i];
+        const NsPlan& pl = P.pl;
+        const muon_mns_problem& f = fused[i];
+        // a tall matrix whose extents need no padding goes into the workspace as it is: a linear pass, partials per chunk
+        const bool linear = P.tall && P.q.rows == pl.Np && P.q.cols == pl.Mp;
+        if (linear != (pass == 0)) continue;
+        MomClass k = {};
+        k.rows = P.q.rows; k.cols = P.q.cols;
+        k.transpose = P.tall ? 0 : 1;
+        k.d_rows = P.tall ? pl.Np : pl.Mp; k.d_cols = P.tall ? pl.Mp : pl.Np;   // padded extents of the matrix itself
+        k.ldd = pl.Mp; k.d_bstride = (long)pl.Mp * pl.Np;
+        k.tiles_x = k.d_cols / MOMLAY_TILE;
+        k.blocks_per_mat = momentum_class_blocks(k, linear ? 1 : 0);
+        k.dst = (uint16_t*)P.Xt[0];
+        k.partial = P.partial;
+        blocks_per_mat[i] = k.blocks_per_mat;
+        int cls = -1;
+        for (int b = 0; b < P.q.batch; ++b) {
+          const bool dtypes_differ = mp.n_mats > 0 && (mp.g_dtype != f.g_dtype || mp.m_dtype != f.m_dtype || mp.w_dtype != f.w_dtype);
+          if (mp.n_mats == MOMG_MAX_MATS || dtypes_differ || (cls < 0 && mp.n_cls == MOMG_MAX_CLS) ||
+              (long)mp.blk_start[mp.n_mats] + k.blocks_per_mat > 0x7ffffff0L) {
+            if ((e = flush()) != hipSuccess) return (int)e;
+            cls = -1;
+          }
+          if (mp.n_mats == 0) {
+            mp.linear = linear ? 1 : 0;
+            mp.g_dtype = f.g_dtype; mp.m_dtype = f.m_dtype; mp.w_dtype = f.w_dtype;
+            mp.c = mc;
+          }
+          if (cls < 0) {
+            cls = mp.n_cls++;
+            mp.cls[cls] = k;
+          }
+          const int j = mp.n_mats++;
+          mp.cls_of[j] = (uint8_t)cls;
+          mp.idx_in_cls[j] = b;
+          mp.blk_start[j + 1] = mp.blk_start[j] + k.blocks_per_mat;
+          mp.g[j] = f.g_ptrs[b];
+          mp.m[j] = f.m_ptrs[b];
+          mp.w[j] = f.w_ptrs ? f.w_ptrs[b] : nullptr;
+          // algorithmic bytes: G read, M read and written, the operand image written (2 bytes each)
+          bytes += (double)P.q.rows * P.q.cols *
+                   ((f.g_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2 * (f.m_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2);
+        }
       }
-      // algorithmic bytes: G read, M read and written, the operand image written (2 bytes each)
-      const double esz = (double)mp.n_mats * P.q.rows * P.q.cols;
-      const double bytes = esz * ((f.g_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2 * (f.m_dtype == MUON_DTYPE_F32 ? 4 : 2) + 2);
-      e = timed_launch(PROF_KEY_MOMENTUM_LAYOUT, bytes, bytes, stream,
-                       [&] { return linear ? launch_momentum_linear(mp, stream) : launch_momentum_layout(mp, stream); });
-      if (e != hipSuccess) return (int)e;
+      if ((e = flush()) != hipSuccess) return (int)e;
     }
-    e = launch_norm_scale_from_partials(P.partial, tiles, P.q.batch, eps, eps_mode, P.scale, stream);
-    if (e != hipSuccess) return (int)e;
+    // 1 / (|U| + eps) of every matrix of every problem from the partial sums: one launch per NORMG_MAX problems
+    NormGroupParams ng = {};
+    for (int i = 0; i <= n_problems; ++i) {
+      if (i == n_problems || ng.n == NORMG_MAX) {
+        if (ng.n > 0 && (e = launch_norm_scale_groups(ng, eps, eps_mode, stream)) != hipSuccess) return (int)e;
+        ng = NormGroupParams{};
+        if (i == n_problems) break;
+      }
+      NormGroup& g = ng.g[ng.n];
+      g.partial = pr[i].partial; g.per_mat = blocks_per_mat[i]; g.scale = pr[i].scale;
+      ng.mat_start[ng.n + 1] = ng.mat_start[ng.n] + pr[i].q.batch;
+      ++ng.n;
+    }
   }
 
   // one product of the iteration for every problem that `fill` accepts: problems that share a tile configuration go

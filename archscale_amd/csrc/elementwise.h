@@ -52,29 +52,53 @@ hipError_t launch_layout_ptrs(const LayoutPtrs& ptrs, int n_mats, int in_dtype, 
                               long d_bstride, int ldd, int d_rows, int d_cols, void* T, long t_bstride, int ldt,
                               hipStream_t stream, float* tile_sumsq);
 
-// momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel)
-constexpr int MOMLAY_MAX = 32;
-constexpr int MOMLAY_TILE = 128;   // rows and columns of the tile of one block; one partial sum per tile
-struct MomLayoutParams {
-  int n_mats, rows, cols;        // matrices of this launch, all rows x cols, contiguous
-  int g_dtype, m_dtype, w_dtype;
+// momentum fused with the layout pass of the Newton-Schulz operand (see momentum_layout_kernel): one launch covers up
+// to MOMG_MAX_MATS matrices (separate allocations: pointers by value) of up to MOMG_MAX_CLS shape classes, either all by
+// the transposing / padding tile pass or all by the linear pass (the operand image is the matrix itself)
+constexpr int MOMG_MAX_MATS = 96;
+constexpr int MOMG_MAX_CLS = 6;
+constexpr int MOMLAY_TILE = 128;   // rows and columns of the tile of one block of the tile pass; one partial sum per tile
+struct MomClass {
+  int rows, cols;                // every matrix of the class is rows x cols, contiguous
   int transpose;                 // dst holds the transpose of the matrix (d_cols x d_rows) instead of the matrix
-  int d_rows, d_cols;            // extents of the matrix padded to multiples of MOMLAY_TILE (the grid)
-  int ldd;                       // leading dimension of dst
+  int d_rows, d_cols;            // tile pass: extents of the matrix padded to multiples of MOMLAY_TILE
+  int ldd;                       // tile pass: leading dimension of dst
+  int blocks_per_mat;            // tiles (tile pass) or chunks of MUON_CHUNK_ELEMS (linear pass) of one matrix
+  int tiles_x;                   // tile pass: tiles along the source columns
   long d_bstride;                // elements between consecutive matrices in dst
-  uint16_t* dst;                 // bf16
-  float* partial;                // [n_mats][(d_rows/MOMLAY_TILE) * (d_cols/MOMLAY_TILE)] sums of squares
-  MomentumCoef c;
-  const void* g[MOMLAY_MAX];
-  void* m[MOMLAY_MAX];
-  const void* w[MOMLAY_MAX];     // read only when c.l2 != 0
+  uint16_t* dst;                 // bf16 image of matrix 0 of the class
+  float* partial;                // [matrices of the class][blocks_per_mat] sums of squares of the values written
 };
-hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream);
-// the case without transposition and padding (dst[mat] laid out like the source): linear chunks of MUON_CHUNK_ELEMS,
-// p.partial = [n_mats][ceil(rows * cols / MUON_CHUNK_ELEMS)]
-hipError_t launch_momentum_linear(const MomLayoutParams& p, hipStream_t stream);
+struct MomGroupParams {
+  int n_mats, n_cls, linear;
+  int g_dtype, m_dtype, w_dtype;
+  MomentumCoef c;
+  MomClass cls[MOMG_MAX_CLS];
+  int32_t blk_start[MOMG_MAX_MATS + 1];   // first block of matrix i of the launch
+  int32_t idx_in_cls[MOMG_MAX_MATS];      // index of matrix i within its class (selects its slot in dst and partial)
+  uint8_t cls_of[MOMG_MAX_MATS];
+  const void* g[MOMG_MAX_MATS];
+  void* m[MOMG_MAX_MATS];
+  const void* w[MOMG_MAX_MATS];           // read only when c.l2 != 0
+};
+static_assert(sizeof(MomGroupParams) <= 4096, "kernel arguments are limited to 4 KiB");
+int momentum_class_blocks(const MomClass& k, int linear);
+hipError_t launch_momentum_group(const MomGroupParams& p, hipStream_t stream);
 hipError_t launch_norm_scale_from_partials(const float* partial, int partials_per_mat, int batch, float eps, int eps_mode,
                                            float* scale, hipStream_t stream);
+// the same for several batches in one launch: block b serves matrix b - mat_start[i] of batch i
+constexpr int NORMG_MAX = 16;
+struct NormGroup {
+  const float* partial;   // [batch][per_mat]
+  float* scale;           // [batch]
+  int per_mat;
+};
+struct NormGroupParams {
+  int n;
+  int32_t mat_start[NORMG_MAX + 1];
+  NormGroup g[NORMG_MAX];
+};
+hipError_t launch_norm_scale_groups(const NormGroupParams& p, float eps, int eps_mode, hipStream_t stream);
 
 hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
                              int batch, int rows, int cols, hipStream_t stream);

@@ -397,19 +397,28 @@ hipError_t launch_layout_ptrs(const LayoutPtrs& ptrs, int n_mats, int in_dtype, 
 //     normalisation 1/(|U| + eps) is applied by the first iteration's GEMM epilogues.  One launch covers up to
 //     MOMLAY_MAX matrices of one shape (their tensors are separate allocations: pointers by value).
 // ---------------------------------------------------------------------------
-// tile of one block: MOMLAY_TILE x MOMLAY_TILE elements, so that a row of it is 256 contiguous bytes in the source and
-// in either destination image
+// tile of one block of the transposing pass: MOMLAY_TILE x MOMLAY_TILE elements (8 elements per thread and pass), so that
+// a row of it is 256 contiguous bytes in the source and in the transposed image.  Measured alternatives (64 x 256,
+// 256 x 64 and 32 x 512 tiles; the loads of all eight passes before the first store) were 5 to 20 % slower.
 constexpr int MOMLAY_TPR = MOMLAY_TILE / 8;          // threads per tile row (8 elements each)
 constexpr int MOMLAY_RPP = 256 / MOMLAY_TPR;         // tile rows per pass of the block
 constexpr int MOMLAY_PASSES = MOMLAY_TILE / MOMLAY_RPP;
 constexpr int MOMLAY_BATCH = 4;                      // passes whose loads are issued before any of their stores
 
+// one matrix of a fused momentum launch, as the block sees it
+struct MomMat {
+  const char* g; char* m; const void* w;
+  int rows, cols, transpose, ldd, w_dtype;
+  uint16_t* dst;      // image of this matrix
+  MomentumCoef c;
+};
+
 template <int GD, int MD>
-__device__ __forceinline__ void momlay_tile(const MomLayoutParams& p, int mat, int r0, int c0,
+__device__ __forceinline__ void momlay_tile(const MomMat& p, int r0, int c0,
                                             uint16_t (&tile)[MOMLAY_TILE][MOMLAY_TILE + 2], float& sumsq) {
-  const char* g = (const char*)p.g[mat];
-  char* m = (char*)p.m[mat];
-  const void* w = p.w[mat];
+  const char* g = p.g;
+  char* m = p.m;
+  const void* w = p.w;
   const int tr = threadIdx.x / MOMLAY_TPR, tc = (threadIdx.x % MOMLAY_TPR) * 8;
   const int c = c0 + tc;
   const bool vec = aligned16(g) && aligned16(m) && (p.cols % 8 == 0) && (p.c.l2 == 0.f || aligned16(w));
@@ -479,28 +488,40 @@ __device__ __forceinline__ void momlay_tile(const MomLayoutParams& p, int mat, i
         u32x4 pk;
         pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
         pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
-        stream_store16(p.dst + (size_t)mat * p.d_bstride + (size_t)r * p.ldd + c, pk);
+        stream_store16(p.dst + (size_t)r * p.ldd + c, pk);
       }
     }
   }
 }
 
+// Tile passes of up to MOMG_MAX_MATS matrices of up to MOMG_MAX_CLS shape classes in ONE launch: block b works on
+// matrix i with blk_start[i] <= b < blk_start[i + 1], on tile b - blk_start[i] of it (tiles along the source columns
+// first).  A class of 32 small matrices alone is a launch of 60 us, a tenth of which is ramp and drain.
 __global__ void __launch_bounds__(256)
-momentum_layout_kernel(const MomLayoutParams p) {
+momentum_layout_kernel(const MomGroupParams p) {
   __shared__ uint16_t tile[MOMLAY_TILE][MOMLAY_TILE + 2];
   __shared__ float red[4];
-  const int mat = blockIdx.z;
-  const int r0 = blockIdx.y * MOMLAY_TILE, c0 = blockIdx.x * MOMLAY_TILE;   // tile of the padded source orientation
+  const int i = find_item(p.blk_start, p.n_mats, blockIdx.x);
+  const int local = blockIdx.x - p.blk_start[i];
+  const MomClass& k = p.cls[p.cls_of[i]];
+  const int idx = p.idx_in_cls[i];
+  const int ty = local / k.tiles_x, tx = local - ty * k.tiles_x;
+  const int r0 = ty * MOMLAY_TILE, c0 = tx * MOMLAY_TILE;   // tile of the padded source orientation
+  MomMat mt;
+  mt.g = (const char*)p.g[i]; mt.m = (char*)p.m[i]; mt.w = p.w[i];
+  mt.rows = k.rows; mt.cols = k.cols; mt.transpose = k.transpose; mt.ldd = k.ldd; mt.w_dtype = p.w_dtype;
+  mt.dst = k.dst + (size_t)idx * k.d_bstride;
+  mt.c = p.c;
   float s[1] = {0.f};
   const int key = (p.g_dtype << 1) | p.m_dtype;
   switch (key) {
-    case 0: momlay_tile<DT_BF16, DT_BF16>(p, mat, r0, c0, tile, s[0]); break;
-    case 1: momlay_tile<DT_BF16, DT_F32>(p, mat, r0, c0, tile, s[0]); break;
-    case 2: momlay_tile<DT_F32, DT_BF16>(p, mat, r0, c0, tile, s[0]); break;
-    default: momlay_tile<DT_F32, DT_F32>(p, mat, r0, c0, tile, s[0]); break;
+    case 0: momlay_tile<DT_BF16, DT_BF16>(mt, r0, c0, tile, s[0]); break;
+    case 1: momlay_tile<DT_BF16, DT_F32>(mt, r0, c0, tile, s[0]); break;
+    case 2: momlay_tile<DT_F32, DT_BF16>(mt, r0, c0, tile, s[0]); break;
+    default: momlay_tile<DT_F32, DT_F32>(mt, r0, c0, tile, s[0]); break;
   }
   __syncthreads();
-  if (p.transpose) {
+  if (mt.transpose) {
     const int tr = threadIdx.x / MOMLAY_TPR, tc = (threadIdx.x % MOMLAY_TPR) * 8;
 #pragma unroll
     for (int h = 0; h < MOMLAY_PASSES; ++h) {
@@ -508,37 +529,30 @@ momentum_layout_kernel(const MomLayoutParams p) {
       const int r = r0 + tc;                    // 8 consecutive columns of it
       uint16_t o[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) o[k] = tile[tc + k][tr + h * MOMLAY_RPP];
+      for (int e = 0; e < 8; ++e) o[e] = tile[tc + e][tr + h * MOMLAY_RPP];
       u32x4 pk;
       pk.x = o[0] | ((uint32_t)o[1] << 16); pk.y = o[2] | ((uint32_t)o[3] << 16);
       pk.z = o[4] | ((uint32_t)o[5] << 16); pk.w = o[6] | ((uint32_t)o[7] << 16);
-      stream_store16(p.dst + (size_t)mat * p.d_bstride + (size_t)c * p.ldd + r, pk);
+      stream_store16(mt.dst + (size_t)c * mt.ldd + r, pk);
     }
   }
   block_reduce<1>(s, red);
-  if (threadIdx.x == 0) p.partial[(size_t)mat * gridDim.x * gridDim.y + blockIdx.y * gridDim.x + blockIdx.x] = s[0];
+  if (threadIdx.x == 0) k.partial[(size_t)idx * k.blocks_per_mat + local] = s[0];
 }
 
-hipError_t launch_momentum_layout(const MomLayoutParams& p, hipStream_t stream) {
-  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.d_rows % MOMLAY_TILE || p.d_cols % MOMLAY_TILE ||
-      p.d_rows / MOMLAY_TILE > 65535 || p.rows > p.d_rows || p.cols > p.d_cols || p.rows < 1 || p.cols < 1)
-    return hipErrorInvalidValue;
-  hipLaunchKernelGGL(momentum_layout_kernel, dim3(p.d_cols / MOMLAY_TILE, p.d_rows / MOMLAY_TILE, p.n_mats), dim3(256), 0,
-                     stream, p);
-  return hipGetLastError();
-}
-
-// The same when the operand image is the matrix itself (no transposition, no padding: dst[mat] has the layout of the
-// source): a linear pass in chunks of MUON_CHUNK_ELEMS like momentum_kernel, one partial sum of squares per chunk.
-// p.d_rows / p.d_cols / p.ldd are not used; p.partial holds [n_mats][chunks_per_mat] values.
+// The same when the operand image is the matrix itself (no transposition, no padding: dst has the layout of the
+// source): linear chunks of MUON_CHUNK_ELEMS like momentum_kernel, one partial sum of squares per chunk.
 __global__ void __launch_bounds__(EW_THREADS)
-momentum_linear_kernel(const MomLayoutParams p, int chunks_per_mat) {
+momentum_linear_kernel(const MomGroupParams p) {
   __shared__ float red[4];
-  const int mat = blockIdx.y, chunk = blockIdx.x;
+  const int i = find_item(p.blk_start, p.n_mats, blockIdx.x);
+  const int chunk = blockIdx.x - p.blk_start[i];
+  const MomClass& k = p.cls[p.cls_of[i]];
+  const int idx = p.idx_in_cls[i];
   PreItem it;
-  it.g = p.g[mat]; it.m = p.m[mat]; it.w = p.w[mat];
-  it.u = p.dst + (size_t)mat * p.d_bstride;
-  it.numel = (long)p.rows * p.cols;
+  it.g = p.g[i]; it.m = p.m[i]; it.w = p.w[i];
+  it.u = k.dst + (size_t)idx * k.d_bstride;
+  it.numel = (long)k.rows * k.cols;
   it.g_dtype = p.g_dtype; it.m_dtype = p.m_dtype; it.u_dtype = DT_BF16; it.w_dtype = p.w_dtype;
   const long begin = (long)chunk * MUON_CHUNK_ELEMS;
   const long end = begin + MUON_CHUNK_ELEMS < it.numel ? begin + MUON_CHUNK_ELEMS : it.numel;
@@ -552,16 +566,37 @@ momentum_linear_kernel(const MomLayoutParams p, int chunks_per_mat) {
     default: momentum_range<DT_F32, DT_F32, DT_BF16, true>(it, begin, end, p.c, vec_ok, &s[0]); break;
   }
   block_reduce<1>(s, red);
-  if (threadIdx.x == 0) p.partial[(size_t)mat * chunks_per_mat + chunk] = s[0];
+  if (threadIdx.x == 0) k.partial[(size_t)idx * k.blocks_per_mat + chunk] = s[0];
 }
 
-hipError_t launch_momentum_linear(const MomLayoutParams& p, hipStream_t stream) {
-  if (p.n_mats < 1 || p.n_mats > MOMLAY_MAX || p.rows < 1 || p.cols < 1 || p.transpose) return hipErrorInvalidValue;
-  const long numel = (long)p.rows * p.cols;
-  if (p.d_bstride < numel) return hipErrorInvalidValue;
-  const long cpm = (numel + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS;
-  if (cpm > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(momentum_linear_kernel, dim3((unsigned)cpm, p.n_mats), dim3(EW_THREADS), 0, stream, p, (int)cpm);
+int momentum_class_blocks(const MomClass& k, int linear) {
+  if (linear) return (int)(((long)k.rows * k.cols + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
+  return (k.d_rows / MOMLAY_TILE) * (k.d_cols / MOMLAY_TILE);
+}
+
+hipError_t launch_momentum_group(const MomGroupParams& p, hipStream_t stream) {
+  if (p.n_mats < 1 || p.n_mats > MOMG_MAX_MATS || p.n_cls < 1 || p.n_cls > MOMG_MAX_CLS || p.blk_start[0] != 0)
+    return hipErrorInvalidValue;
+  for (int c = 0; c < p.n_cls; ++c) {
+    const MomClass& k = p.cls[c];
+    if (k.rows < 1 || k.cols < 1 || !k.dst || !k.partial || k.blocks_per_mat != momentum_class_blocks(k, p.linear))
+      return hipErrorInvalidValue;
+    if (p.linear) {
+      if (k.transpose || k.d_bstride < (long)k.rows * k.cols) return hipErrorInvalidValue;
+    } else if (k.d_rows % MOMLAY_TILE || k.d_cols % MOMLAY_TILE || k.rows > k.d_rows || k.cols > k.d_cols ||
+               k.tiles_x != k.d_cols / MOMLAY_TILE) {
+      return hipErrorInvalidValue;
+    }
+  }
+  // every block must decode to a tile (chunk) inside its matrix
+  for (int i = 0; i < p.n_mats; ++i) {
+    if (p.cls_of[i] >= p.n_cls || !p.g[i] || !p.m[i] || (p.c.l2 != 0.f && !p.w[i])) return hipErrorInvalidValue;
+    if (p.blk_start[i + 1] - p.blk_start[i] != p.cls[p.cls_of[i]].blocks_per_mat) return hipErrorInvalidValue;
+  }
+  const int blocks = p.blk_start[p.n_mats];
+  if (blocks <= 0) return hipErrorInvalidValue;
+  if (p.linear) hipLaunchKernelGGL(momentum_linear_kernel, dim3(blocks), dim3(EW_THREADS), 0, stream, p);
+  else hipLaunchKernelGGL(momentum_layout_kernel, dim3(blocks), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -571,6 +606,29 @@ hipError_t launch_norm_scale_from_partials(const float* partial, int partials_pe
   if (batch < 1 || partials_per_mat < 1) return hipErrorInvalidValue;
   hipLaunchKernelGGL(norm_scale_kernel, dim3(batch), dim3(EW_THREADS), 0, stream, partial, partials_per_mat, eps, eps_mode,
                      scale, (float*)nullptr);
+  return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+norm_scale_groups_kernel(const NormGroupParams p, float eps, int eps_mode) {
+  __shared__ float red[4];
+  const int i = find_item(p.mat_start, p.n, blockIdx.x);
+  const NormGroup& g = p.g[i];
+  const int b = blockIdx.x - p.mat_start[i];
+  float s[1] = {0.f};
+  for (int t = threadIdx.x; t < g.per_mat; t += EW_THREADS) s[0] += g.partial[(size_t)b * g.per_mat + t];
+  block_reduce<1>(s, red);
+  if (threadIdx.x == 0) {
+    const float n = sqrtf(s[0]);
+    g.scale[b] = eps_mode == EPS_ADD ? 1.f / (n + eps) : 1.f / fmaxf(n, eps);
+  }
+}
+
+hipError_t launch_norm_scale_groups(const NormGroupParams& p, float eps, int eps_mode, hipStream_t stream) {
+  if (p.n < 1 || p.n > NORMG_MAX || p.mat_start[0] != 0) return hipErrorInvalidValue;
+  for (int i = 0; i < p.n; ++i)
+    if (!p.g[i].partial || !p.g[i].scale || p.g[i].per_mat < 1 || p.mat_start[i + 1] <= p.mat_start[i]) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(norm_scale_groups_kernel, dim3(p.mat_start[p.n]), dim3(EW_THREADS), 0, stream, p, eps, eps_mode);
   return hipGetLastError();
 }
 

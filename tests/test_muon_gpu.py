@@ -150,6 +150,7 @@ def test_hook_state_dict_and_groups(gpu_device):
     from archscale_amd.optim.muon import Muon
     import archscale_amd.optim.newton_schulz_hip as H
     shapes = [(64, 128), (128, 64)]
+    torch.manual_seed(4)      # the device-side draws below: the same values whichever tests ran before this one
     params = _make(shapes, torch.float32, 4, gpu_device)
     vec = torch.nn.Parameter(torch.randn(128, device=gpu_device))
     emb = torch.nn.Parameter(torch.randn(50, 64, device=gpu_device))
