@@ -27,15 +27,18 @@ struct NsPlan {
   int m, n;      // short / long side of a matrix
   int Mp, Np;    // padded to the tile
   int cpm;       // norm chunks per matrix
-  size_t off_xt[2], off_a, off_bh, off_bl, off_partial, off_scale, total;
+  size_t off_xt[2], off_a, off_bh, off_bl, off_partial, off_scale, off_skpart, off_skcnt, total;
+  int sk_quadrants;   // K-split: 128x128 quadrants per matrix that have partial results (0: none)
 };
 
 // The ARCHSCALE_MUON_* environment is read ONCE, when the first call needs it (debugging switches: a tile configuration
-// forced for every problem, the quartered last round switched off); later changes of the environment are not seen.
+// forced for every problem, the quartered last round or the K-split switched off); later changes are not seen.
 struct EnvSwitches {
   int tile;       // 0, 128 or 256
   bool quarter;
-  EnvSwitches() : tile(0), quarter(true) {
+  int ksplit;     // 0: no K-split
+  EnvSwitches() : tile(0), quarter(true), ksplit(1) {
+    if (const char* k = getenv("ARCHSCALE_MUON_KSPLIT")) ksplit = atoi(k);   // 0: off; 2, 4, 8: that many parts wherever the rule splits
     if (const char* t = getenv("ARCHSCALE_MUON_TILE")) {
       const int v = atoi(t);
       if (v == 128 || v == 256) tile = v;
@@ -58,13 +61,50 @@ int pick_tile(int m, int n) {
   return cost(256, 1.0) <= cost(128, 1.25) ? 256 : 128;
 }
 
+inline long sym_tiles(int t) { return (long)t * (t + 1) / 2; }
+
+// K-split of a symmetric product of ONE matrix, a pure function of the matrix's own shape (so a matrix takes the same
+// path, and gives the same bits, alone and in any batch).  With tm = tiles of 256 along the short side and KT k-tiles of
+// 64: the first `full` = floor(T / 256) * 256 upper-triangle tiles (whole rounds of the chip when the matrix is alone)
+// run as they are; the remaining `rem` run as 128x128 quadrants, `parts` blocks per quadrant, each walking KT / parts
+// k-tiles.  Only long reductions (KT >= 128, i.e. K >= 8192) of matrices with at least 16 tiles left over are split: the
+// partial results cost 64 KiB of traffic per block each way, which a block of 32 or more k-tiles hides, and a batch of
+// many small matrices (whose launches are full anyway) must not pay for it.  Measured on single matrices (us per
+// product, 2 / 4 / 8 parts against none): the 136 tiles of a 4096 x 14336 matrix 330 / 315 / 366 against 378, the 16 tiles
+// left over by an 8192 x 8192 matrix 55 / 40 / 43 against 83; a batch of eight 8192 x 8192 matrices, which needs no split,
+// pays 1.5 % of its time for the partial results.
+struct SkRule { int full, rem, parts; };
+constexpr int SK_PARTS = 4, SK_MIN_KT = 128, SK_MIN_REM = 16;
+SkRule sk_rule(int tm, int KT) {
+  const int T = (int)sym_tiles(tm);
+  SkRule r = {T, 0, 1};
+  const int full = T / 256 * 256, rem = T - full;
+  if (env_switches().ksplit == 0 || KT < SK_MIN_KT || rem < SK_MIN_REM) return r;
+  int parts = SK_PARTS;
+  if (env_switches().ksplit > 1 && KT / env_switches().ksplit >= 16) parts = env_switches().ksplit;   // (experiments)
+  return SkRule{full, rem, parts};
+}
+// the two reduction lengths of a matrix's symmetric products: the long side (A = X X^T) and the short side (the m x m products)
+struct SkShape { SkRule long_k, short_k; bool any; };
+SkShape sk_shape(int m, int n) {
+  const int tm = (int)(round_up(m, 256) / 256);
+  SkShape s;
+  s.long_k = sk_rule(tm, (int)(round_up(n, 256) / 64));
+  s.short_k = sk_rule(tm, (int)(round_up(m, 256) / 64));
+  s.any = s.long_k.rem > 0 || s.short_k.rem > 0;
+  return s;
+}
+
 NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   NsPlan p;
   p.m = rows < cols ? rows : cols;
   p.n = rows < cols ? cols : rows;
   p.tile = tile ? tile : pick_tile(p.m, p.n);
-  p.Mp = (int)round_up(p.m, p.tile);
-  p.Np = (int)round_up(p.n, p.tile);
+  const SkShape sk = sk_shape(p.m, p.n);
+  // a shape with a K-split is enumerated in tiles of 256 whatever the configuration of the call
+  const int pad = sk.any ? 256 : p.tile;
+  p.Mp = (int)round_up(p.m, pad);
+  p.Np = (int)round_up(p.n, pad);
   p.cpm = (int)(((long)rows * cols + MUON_CHUNK_ELEMS - 1) / MUON_CHUNK_ELEMS);
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off = (size_t)round_up((long)(off + bytes), 256); return o; };
@@ -81,11 +121,14 @@ NsPlan make_plan(int batch, int rows, int cols, int prec_mode, int tile = 0) {
   const size_t tiles64 = (size_t)(p.Mp / 64) * (p.Np / 64);
   p.off_partial = take((size_t)batch * std::max((size_t)p.cpm, tiles64) * sizeof(float));
   p.off_scale = take((size_t)2 * batch * sizeof(float));   // deferred factor and the power of two applied to the copy
+  // K-split: fp32 partial results ([matrix][quadrant][part]) and one counter per quadrant
+  p.sk_quadrants = 4 * std::max(sk.long_k.rem, sk.short_k.rem);
+  const int parts = std::max(sk.long_k.rem ? sk.long_k.parts : 0, sk.short_k.rem ? sk.short_k.parts : 0);
+  p.off_skpart = take((size_t)batch * p.sk_quadrants * parts * SK_TILE_BYTES);
+  p.off_skcnt = take((size_t)batch * p.sk_quadrants * sizeof(int));
   p.total = off;
   return p;
 }
-
-inline long sym_tiles(int t) { return (long)t * (t + 1) / 2; }
 // matrix-core work of the upper-triangle tiles, in tiles: a diagonal tile runs three quarters of its MFMAs (the waves
 // whose sub-tiles lie wholly below the diagonal sit out)
 inline double sym_tiles_issued(int t) { return (double)sym_tiles(t) - 0.25 * t; }
@@ -260,6 +303,8 @@ struct NsProblem {
   NsPlan pl;
   __bf16 *Xt[2], *A, *Bh, *Bl;   // Xt: the iterate as X^T, [b][Np][Mp] (long side first), ping-pong
   float *partial, *scale, *pow2;
+  float* sk_partial;   // K-split: partial results and counters (null when the shape has none)
+  int* sk_counter;
   bool tall;
   bool gram_tail;   // the last two iterations run on the Gram side (n >= 2m): one B X product instead of two
   bool defer;   // the operand of the first iteration is the input as it is; its epilogues apply 1/(|X| + eps)
@@ -342,6 +387,8 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     P.partial = (float*)(ws + P.pl.off_partial);
     P.scale = (float*)(ws + P.pl.off_scale);
     P.pow2 = P.scale + P.q.batch;
+    P.sk_partial = P.pl.sk_quadrants ? (float*)(ws + P.pl.off_skpart) : nullptr;
+    P.sk_counter = P.pl.sk_quadrants ? (int*)(ws + P.pl.off_skcnt) : nullptr;
     // a square matrix counts as tall: orthogonalising X^T and transposing the result is the same map, and a tall
     // matrix enters the workspace as it is (a linear pass instead of a tile transpose)
     P.tall = P.q.rows >= P.q.cols;
@@ -369,8 +416,11 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
     return (long)pr[a].pl.Mp * pr[a].pl.Np > (long)pr[b].pl.Mp * pr[b].pl.Np;
   });
 
-  // normalise into X^T (long side first): a wide input is transposed on the way, a tall one is copied as it is
   hipError_t e;
+  // K-split counters start at zero (every launch leaves them at zero again); the workspace is the caller's and holds anything
+  for (const NsProblem& P : pr)
+    if (P.sk_counter && (e = launch_zero_i32(P.sk_counter, (long)P.q.batch * P.pl.sk_quadrants, stream)) != hipSuccess) return (int)e;
+  // normalise into X^T (long side first): a wide input is transposed on the way, a tall one is copied as it is
   for (int i = 0; i < n_problems && !fused; ++i) {
     const NsProblem& P = pr[i];
     const NsPlan& pl = P.pl;
@@ -472,6 +522,23 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   // one product of the iteration for every problem that `fill` accepts: problems that share a tile configuration go
   // into one launch (at most MAX_GROUPS per launch)
   auto run_mode = [&](int mode, bool split_launch, bool final_, int ws16, auto&& fill) -> hipError_t {
+    const bool sym = mode != MODE_BX;
+    // tiles of symmetric products that take a K-split (see sk_rule), of every problem: one launch of its own
+    GroupedGemmParams sk = {};
+    sk.quarter = 1;
+    double sk_fa = 0.0, sk_fi = 0.0;
+    auto flush_sk = [&]() -> hipError_t {
+      if (sk.n_groups == 0) return hipSuccess;
+      const int key = 128 * 100 + mode * 10;
+      const GroupedGemmParams launch = sk;
+      hipError_t err = timed_launch(key, sk_fa, sk_fi, stream, [&] {
+        return launch_ns_gemm_grouped(128, mode, false, false, launch, stream, ws16, true);
+      });
+      sk = GroupedGemmParams{};
+      sk.quarter = 1;
+      sk_fa = sk_fi = 0.0;
+      return err;
+    };
     for (int tile : {256, 128}) {
       GroupedGemmParams gp = {};
       double fa = 0.0, fi = 0.0;
@@ -488,7 +555,36 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
         GemmParams g = {};
         double a_fl = 0.0, i_fl = 0.0;
         if (!fill(P, g, a_fl, i_fl)) continue;
-        const long tiles = ns_gemm_tiles(mode, g);
+        long tiles = ns_gemm_tiles(mode, g);
+        if (sym && P.pl.sk_quadrants > 0 && !split_launch) {
+          // the shape has a K-split for some reduction length: this product's own rule, in tiles of 256
+          const SkRule r = sk_rule(P.pl.Mp / 256, g.K / 64);
+          if (r.rem > 0) {
+            GemmParams q = g;
+            q.tilesM = q.tilesN = P.pl.Mp / 128;          // quarter mode counts the fine tiles
+            q.qt_first = 0;
+            q.t_first = r.full; q.t_count = r.rem;
+            q.ksplit = r.parts;
+            q.sk_partial = P.sk_partial; q.sk_counter = P.sk_counter;
+            const long blocks = 4L * g.batch * r.rem * r.parts;
+            if (blocks + sk.tile_start[sk.n_groups] > 0x7ffffff0L || sk.n_groups == MAX_GROUPS) {
+              hipError_t err = flush_sk();
+              if (err != hipSuccess) return err;
+            }
+            if (blocks > 0x7ffffff0L) return hipErrorInvalidValue;
+            sk.g[sk.n_groups] = q;
+            sk.tile_start[sk.n_groups + 1] = sk.tile_start[sk.n_groups] + (int)blocks;
+            ++sk.n_groups;
+            const double share = (double)r.rem / (r.full + r.rem);
+            sk_fa += a_fl * share; sk_fi += i_fl * share;
+            a_fl *= 1.0 - share; i_fl *= 1.0 - share;
+            if (r.full == 0) continue;
+            // the whole rounds run as they are; a forced small configuration never gets here (it has fewer than 128 tiles)
+            if (tile != 256) return hipErrorInvalidValue;
+            g.t_first = 0; g.t_count = r.full;
+            tiles = (long)g.batch * r.full;
+          }
+        }
         if (tiles + gp.tile_start[gp.n_groups] > 0x7ffffff0L || gp.n_groups == MAX_GROUPS) {
           hipError_t err = flush();
           if (err != hipSuccess) return err;
@@ -503,7 +599,7 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
       hipError_t err = flush();
       if (err != hipSuccess) return err;
     }
-    return hipSuccess;
+    return flush_sk();
   };
 
   // ---- storage of the iteration's matrices, per iteration.  MUON_PREC_F16: half from the first iteration on, or from

@@ -100,6 +100,9 @@ struct NormGroupParams {
 };
 hipError_t launch_norm_scale_groups(const NormGroupParams& p, float eps, int eps_mode, hipStream_t stream);
 
+// p[0 .. n) <- 0 with a plain kernel (a launch that a graph capture records like any other)
+hipError_t launch_zero_i32(int* p, long n, hipStream_t stream);
+
 hipError_t launch_unpad_copy(const void* src, long s_bstride, int lds_, void* dst, long d_bstride, int ldd,
                              int batch, int rows, int cols, hipStream_t stream);
 

@@ -632,6 +632,17 @@ hipError_t launch_norm_scale_groups(const NormGroupParams& p, float eps, int eps
   return hipGetLastError();
 }
 
+__global__ void __launch_bounds__(256) zero_i32_kernel(int* __restrict__ p, long n) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+hipError_t launch_zero_i32(int* p, long n, hipStream_t stream) {
+  if (!p || n <= 0 || n > 0x7fffffffL * 256) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(zero_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, n);
+  return hipGetLastError();
+}
+
 // strided copy of the leading rows x cols corner of a padded bf16 buffer into a caller tensor
 __global__ void __launch_bounds__(256)
 unpad_copy_kernel(const uint16_t* __restrict__ src, long s_bstride, int lds_, uint16_t* __restrict__ dst,

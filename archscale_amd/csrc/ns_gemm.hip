@@ -77,10 +77,14 @@ __device__ __forceinline__ int lds_chunk_off(int r, int c) { return r * ROW_BYTE
 // F16 = 1: the workspace matrices (operands, addend, non-final outputs) are IEEE half instead of bfloat16 (the caller's
 // tensors stay bfloat16); the host keeps them in range with power-of-two factors folded into alpha / beta / out_shift.
 // F16 = 2: bfloat16 operands and addend, IEEE-half output (the step from a bfloat16 iteration to a half one).
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND, int F16>
+// SK: problems of the launch may carry a K-split (GemmParams::ksplit; symmetric products, 128x128 configuration): the
+// blocks that share a tile leave their fp32 accumulators in the workspace and the last one to arrive adds them up in
+// the order of the parts and runs the epilogue.
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND, int F16, bool SK>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
 ns_gemm_kernel(const GroupedGemmParams gp) {
   static_assert(!(F16 && SPLIT), "the hi+lo pair is a bfloat16 device");
+  static_assert(!SK || (BM == 128 && !SPLIT && !FINAL && MODE != MODE_BX), "the K-split serves symmetric products in the small configuration");
   static_assert(F16 != 2 || (MODE == MODE_BX && !FINAL), "only X' changes its storage type");
   constexpr bool IN16 = F16 == 1, OUT16 = F16 != 0;
   constexpr int NW = (BM / WM) * (BN / WN);
@@ -124,6 +128,13 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   while (grp + 1 < gp.n_groups && logical >= gp.tile_start[grp + 1]) ++grp;
   const GemmParams p = gp.g[grp];
   int local = logical - gp.tile_start[grp];
+  int ks = 0;   // part of the K range this block walks
+  if constexpr (SK) {
+    const int launch_tiles = (gp.tile_start[grp + 1] - gp.tile_start[grp]) / p.ksplit;
+    ks = local / launch_tiles;
+    local -= ks * launch_tiles;
+  }
+  const int sk_tile = local;   // this tile among the problem's tiles in the launch
   // grid the tile index is decoded in: the problem's own, or the 2x coarser one whose tiles this launch quarters
   int dM = p.tilesM, dN = p.tilesN, quadrant = 0;
   if (gp.quarter) {
@@ -133,8 +144,10 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     dN >>= 1;
   }
   const int tiles_per_mat = SYM ? (dM * (dM + 1)) / 2 : dM * dN;
-  const int b = local / tiles_per_mat;
-  int t = local - b * tiles_per_mat;
+  // the launch may cover only tiles [t_first, t_first + t_count) of every matrix
+  const int per_mat = p.t_count > 0 ? p.t_count : tiles_per_mat;
+  const int b = local / per_mat;
+  int t = p.t_first + (local - b * per_mat);
   int ti, tj;
   if (SYM) {
     ti = 0;
@@ -157,6 +170,14 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const char* P2b = KSPLIT ? (const char*)(p.P2 + (size_t)b * p.strideP + (size_t)R0 * p.ldp) : nullptr;
   const char* Qb = KMAJ ? (const char*)(p.Q + (size_t)b * p.strideQ + C0)
                         : (const char*)(p.Q + (size_t)b * p.strideQ + (size_t)C0 * p.ldq);
+  int KT = p.K / BK;
+  if constexpr (SK) {
+    // part ks of ksplit: k-tiles [ks KT / ksplit, (ks + 1) KT / ksplit), at least one (the host checks KT >= ksplit)
+    const int kt0 = (int)((long)ks * KT / p.ksplit), kt1 = (int)((long)(ks + 1) * KT / p.ksplit);
+    Pb += KMAJ ? (size_t)kt0 * BK * p.ldp * 2 : (size_t)kt0 * ROW_BYTES;
+    Qb += KMAJ ? (size_t)kt0 * BK * p.ldq * 2 : (size_t)kt0 * ROW_BYTES;
+    KT = kt1 - kt0;
+  }
 
   // per-lane byte offsets of the global chunks this lane copies (k-tile 0)
   uint32_t offP[JP], offQ[JQ];
@@ -189,7 +210,6 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     }
   }
 
-  const int KT = p.K / BK;
   const int KT_ALL = KSPLIT ? 2 * KT : KT;
 
   // copy j (of JP + JQ per wave) of k-tile kt: one 1 KiB slab (8 rows x 128 B) straight into stage kt & 1
@@ -338,32 +358,47 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   using C3 = std::integral_constant<int, G3>;
   using C4 = std::integral_constant<int, NGL>;
   // k-steps 0..2 of k-tile kt (with the rest of the copies of kt+1), barrier, k-step 3 (with the first
-  // copies of kt+2).  COPY_REST / NEXT / COPY_FIRST: k-tiles kt+1 / kt+1 / kt+2 exist.
-  auto ktile = [&](int kt, auto copy_rest, auto next, auto copy_first) {
+  // copies of kt+2).  COPY_REST / NEXT / COPY_FIRST: k-tiles kt+1 / kt+1 / kt+2 exist.  ACTIVE = false is the same
+  // sequence of copies, waits and barriers without the fragment reads and the MFMAs: what a wave runs whose sub-tile
+  // lies below the diagonal of a symmetric product (one code path, so the barriers of the two kinds of wave cannot
+  // drift apart).
+  auto ktile = [&](int kt, auto copy_rest, auto next, auto copy_first, auto active) {
     constexpr bool COPY_REST = decltype(copy_rest)::value, NEXT = decltype(next)::value, COPY_FIRST = decltype(copy_first)::value;
+    using Act = std::integral_constant<bool, decltype(active)::value>;
     const char* sP = smem + (kt & 1) * STAGE;
     const char* sQ = sP + PBYTES;
     const char* nP = smem + ((kt + 1) & 1) * STAGE;
     const char* nQ = nP + PBYTES;
     if constexpr (COPY_REST) {
-      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I1{}, kt + 1, C1{}, C2{});
-      phase(Yes{}, Yes{}, I1{}, I0{}, sP, sQ, I2{}, kt + 1, C2{}, C3{});
-      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I3{}, kt + 1, C3{}, C4{});
+      phase(Act{}, Act{}, I0{}, I1{}, sP, sQ, I1{}, kt + 1, C1{}, C2{});
+      phase(Act{}, Act{}, I1{}, I0{}, sP, sQ, I2{}, kt + 1, C2{}, C3{});
+      phase(Act{}, Act{}, I0{}, I1{}, sP, sQ, I3{}, kt + 1, C3{}, C4{});
     } else {
-      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I1{}, 0, I0{}, I0{});
-      phase(Yes{}, Yes{}, I1{}, I0{}, sP, sQ, I2{}, 0, I0{}, I0{});
-      phase(Yes{}, Yes{}, I0{}, I1{}, sP, sQ, I3{}, 0, I0{}, I0{});
+      phase(Act{}, Act{}, I0{}, I1{}, sP, sQ, I1{}, 0, I0{}, I0{});
+      phase(Act{}, Act{}, I1{}, I0{}, sP, sQ, I2{}, 0, I0{}, I0{});
+      phase(Act{}, Act{}, I0{}, I1{}, sP, sQ, I3{}, 0, I0{}, I0{});
     }
     if constexpr (NEXT) {
       // this wave's copies of kt+1 have landed and its reads of kt are done; after the barrier that holds for all
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (COPY_FIRST) phase(Yes{}, Yes{}, I1{}, I0{}, nP, nQ, I0{}, kt + 2, I0{}, C1{});
-      else phase(Yes{}, Yes{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
+      if constexpr (COPY_FIRST) phase(Act{}, Act{}, I1{}, I0{}, nP, nQ, I0{}, kt + 2, I0{}, C1{});
+      else phase(Act{}, Act{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
     } else {
-      phase(Yes{}, No{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
+      phase(Act{}, No{}, I1{}, I0{}, nP, nQ, I0{}, 0, I0{}, I0{});
     }
+  };
+  // the whole K range: ACTIVE waves multiply, the others only copy and meet the barriers
+  auto k_range = [&](auto active) {
+    using Act = std::integral_constant<bool, decltype(active)::value>;
+    if constexpr (Act::value) {
+#pragma unroll
+      for (int r = 0; r < NRD; ++r) fread(0, smem, smem + PBYTES, 0, r);
+    }
+    for (int kt = 0; kt + 2 < KT_ALL; ++kt) ktile(kt, Yes{}, Yes{}, Yes{}, Act{});
+    if (KT_ALL > 1) ktile(KT_ALL - 2, Yes{}, Yes{}, No{}, Act{});
+    ktile(KT_ALL - 1, No{}, No{}, No{}, Act{});
   };
 
 #pragma unroll
@@ -379,27 +414,8 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
-  if (!idle) {
-#pragma unroll
-    for (int r = 0; r < NRD; ++r) fread(0, smem, smem + PBYTES, 0, r);
-    for (int kt = 0; kt + 2 < KT_ALL; ++kt) ktile(kt, Yes{}, Yes{}, Yes{});
-    if (KT_ALL > 1) ktile(KT_ALL - 2, Yes{}, Yes{}, No{});
-    ktile(KT_ALL - 1, No{}, No{}, No{});
-  } else {
-    // an idle wave keeps its share of the copies and meets every barrier of the loop above (one per k-tile that has a
-    // successor), in the same order: rest of k-tile kt+1, barrier, first copies of k-tile kt+2
-    for (int kt = 0; kt + 1 < KT_ALL; ++kt) {
-#pragma unroll
-      for (int g = G1; g < NGL; ++g) gload(kt + 1, g);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      if (kt + 2 < KT_ALL) {
-#pragma unroll
-        for (int g = 0; g < G1; ++g) gload(kt + 2, g);
-      }
-    }
-  }
+  if (!idle) k_range(Yes{});
+  else k_range(No{});
 
   // ---- epilogue.  acc[i][j][e] of lane l is element
   //   rl = wr0 + i*32 + 8*(e/4) + 4*(l/32) + e%4  (row in the tile),   cl = wc0 + j*32 + l%32  (column)
@@ -413,6 +429,57 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   // partial-line requests and cost a quarter of the kernel.
   static_assert(BM == BN, "square block tiles");
   constexpr int NT = NW * 64;
+  if constexpr (SK) {
+    if (p.ksplit > 1) {
+      // Every part leaves its accumulators in the workspace (accumulator layout: one word per lane and accumulator
+      // register, so every access of a wave is a run of 256 bytes), waits until they have arrived, and counts itself in.
+      // The block that finds itself last adds ALL parts in the order 0, 1, ... (its own from memory like the others: the
+      // sum of a tile is the same whichever block came last) and goes on to the epilogue; the others are done.  Nobody
+      // waits for anybody.  The partial results travel as system-scope accesses (written through, read past the
+      // caches): the eight L2 caches of the chip are not coherent with each other, and the alternative - a release /
+      // acquire fence per block - writes back and invalidates a whole L2 each time (measured: the product twice as slow).
+      __shared__ int sk_last;
+      float* part = p.sk_partial + (size_t)sk_tile * p.ksplit * (BM * BN);
+      if (!idle) {
+        float* dst = part + (size_t)ks * (BM * BN);
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              __hip_atomic_store(dst + ((i * FN + j) * 16 + e) * NT + tid, acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's stores have been acknowledged
+      __syncthreads();
+      if (tid == 0) {
+        const int old = __hip_atomic_fetch_add(p.sk_counter + sk_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = old == p.ksplit - 1;
+        if (last) __hip_atomic_store(p.sk_counter + sk_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+        sk_last = last;
+      }
+      __syncthreads();
+      if (!sk_last) return;
+      if (!idle) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int sidx = 0; sidx < p.ksplit; ++sidx) {
+          const float* src = part + (size_t)sidx * (BM * BN);
+#pragma unroll
+          for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+              for (int e = 0; e < 16; ++e)
+                acc[i][j][e] += __hip_atomic_load(src + ((i * FN + j) * 16 + e) * NT + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+      }
+    }
+  }
   constexpr int TPITCH = BN * 2;            // bytes per staged row (both images)
   constexpr int CPRT = BN / 8;              // 16-byte chunks per staged row
   constexpr int PASSES = (BM * BN / 8) / NT;
@@ -784,11 +851,11 @@ long ns_gemm_tiles(int mode, const GemmParams& p) {
   return (long)p.batch * (sym ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN);
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true, int F16 = 0>
+template <int BM, int BN, int WM, int WN, int MODE, bool SPLIT, bool FINAL, bool ADDEND = true, int F16 = 0, bool SK = false>
 static hipError_t launch_one(const GroupedGemmParams& gp, hipStream_t stream) {
   constexpr int NT = (BM / WM) * (BN / WN) * 64;
   constexpr int SMEM = 2 * (BM + BN) * ROW_BYTES;
-  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>;
+  auto kern = ns_gemm_kernel<BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16, SK>;
   // the dynamic-LDS limit is an attribute of the function on ONE device: set it once per device and instantiation
   // (the call is idempotent, so two threads that race on the first launch only repeat it)
   static std::atomic<bool> attr_set[64];
@@ -846,25 +913,54 @@ static hipError_t launch_cfg(int mode, bool split, bool final_, const GroupedGem
   }
 }
 
+// the symmetric products of the 128x128 configuration with a K-split
+template <int F16>
+static hipError_t launch_ksplit(int mode, const GroupedGemmParams& p, hipStream_t s) {
+  switch (mode) {
+    case MODE_SYRK: return launch_one<128, 128, 64, 64, MODE_SYRK, false, false, true, F16, true>(p, s);
+    case MODE_SYRKT: return launch_one<128, 128, 64, 64, MODE_SYRKT, false, false, true, F16, true>(p, s);
+    case MODE_SYRK2: return launch_one<128, 128, 64, 64, MODE_SYRK2, false, false, true, F16, true>(p, s);
+  }
+  return hipErrorInvalidValue;
+}
+
 hipError_t launch_ns_gemm_grouped(int tile, int mode, bool split, bool final_, const GroupedGemmParams& gp,
-                                  hipStream_t stream, int f16) {
+                                  hipStream_t stream, int f16, bool ksplit) {
   if (gp.n_groups < 1 || gp.n_groups > MAX_GROUPS) return hipErrorInvalidValue;
   const bool sym = (mode == MODE_SYRK || mode == MODE_SYRK2 || mode == MODE_SYRKT);
+  if (ksplit && (!sym || tile != 128 || split || final_ || f16 == 2)) return hipErrorInvalidValue;
   for (int i = 0; i < gp.n_groups; ++i) {
     const GemmParams& g = gp.g[i];
     if (g.K % BK != 0 || g.K <= 0 || gp.tile_start[i + 1] < gp.tile_start[i]) return hipErrorInvalidValue;
     if (mode == MODE_SYRK2 && !g.E) return hipErrorInvalidValue;
     if (mode == MODE_BX && (g.E == nullptr) != (gp.g[0].E == nullptr)) return hipErrorInvalidValue;  // one kernel per launch
+    long blocks = (long)gp.tile_start[i + 1] - gp.tile_start[i];
+    if (!ksplit) {
+      if (g.ksplit > 1) return hipErrorInvalidValue;
+    } else {
+      // every part walks at least one k-tile; the parts of a tile find their partial results and their counter
+      if (g.ksplit < 1 || g.ksplit > g.K / BK || blocks % g.ksplit) return hipErrorInvalidValue;
+      if (g.ksplit > 1 && (!g.sk_partial || !g.sk_counter || ((uintptr_t)g.sk_partial & 15))) return hipErrorInvalidValue;
+      blocks /= g.ksplit;
+    }
     // every block must decode to a tile inside the problem
-    const long blocks = (long)gp.tile_start[i + 1] - gp.tile_start[i];
+    if (g.t_first < 0 || g.t_count < 0 || (g.t_count == 0 && g.t_first != 0)) return hipErrorInvalidValue;
     if (!gp.quarter) {
-      if (blocks > ns_gemm_tiles(mode, g)) return hipErrorInvalidValue;
+      const long per = ns_gemm_tiles(mode, g) / g.batch;
+      if (g.t_count ? (g.t_first + g.t_count > per || blocks > (long)g.batch * g.t_count) : blocks > ns_gemm_tiles(mode, g))
+        return hipErrorInvalidValue;
     } else {
       if ((g.tilesM & 1) || (!sym && (g.tilesN & 1)) || g.qt_first < 0 || (blocks & 3)) return hipErrorInvalidValue;
       const long cm = g.tilesM / 2, cn = g.tilesN / 2;
-      const long coarse = (long)g.batch * (sym ? cm * (cm + 1) / 2 : cm * cn);
+      const long per = sym ? cm * (cm + 1) / 2 : cm * cn;
+      if (g.t_count && g.t_first + g.t_count > per) return hipErrorInvalidValue;
+      const long coarse = (long)g.batch * (g.t_count ? g.t_count : per);
       if (g.qt_first + blocks / 4 > coarse) return hipErrorInvalidValue;
     }
+  }
+  if (ksplit) {
+    if (f16 == 1) return launch_ksplit<1>(mode, gp, stream);
+    return launch_ksplit<0>(mode, gp, stream);
   }
   if (f16 == 1) {
     if (tile == 256) return launch_cfg<256, 256, 128, 64, 1>(mode, split, final_, gp, stream);

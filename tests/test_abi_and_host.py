@@ -254,8 +254,8 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             found |= set(range(int(a), int(b) + 1)) if a else {int(c)}
         return found
 
-    # template arguments of an instantiation from its mangled name: <BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16>
-    targs = re.compile(r"ns_gemm_kernelILi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])ELb([01])ELi(\d+)EE")
+    # template arguments of an instantiation from its mangled name: <BM, BN, WM, WN, MODE, SPLIT, FINAL, ADDEND, F16, SK>
+    targs = re.compile(r"ns_gemm_kernelILi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])ELb([01])ELi(\d+)ELb([01])EE")
     # pass 1: cut every K-major instantiation into basic blocks (label -> instructions, each tagged "inline asm or not")
     seen, reads_of, kernels = set(), {}, {}
     all_kernels = 0
@@ -269,9 +269,9 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             m = targs.search(code)
             assert m, f"cannot read the template arguments of {code}: the name mangling changed, adapt this test"
             all_kernels += 1
-            bm, mode, f16 = int(m.group(1)), int(m.group(5)), int(m.group(9))
+            bm, mode, f16, sk = int(m.group(1)), int(m.group(5)), int(m.group(9)), int(m.group(10))
             inside = mode == 3                   # MODE_SYRKT instantiations
-            cur = (bm, f16)
+            cur = (bm, f16, sk)
             if inside:
                 assert cur not in seen, f"{code} seen twice"
                 seen.add(cur)
@@ -342,9 +342,10 @@ def test_transpose_read_results_are_not_touched_before_the_explicit_wait(tmp_pat
             out = walk(instrs, pend_in[i], True, key)
             if instrs and instrs[-1][0].startswith("s_endpgm"):
                 assert not out, f"{key}: transpose reads in flight at the end of the program"
-    # every K-major instantiation was visited by name: two tile configurations x {bfloat16, half} workspace
-    assert seen == {(256, 0), (256, 1), (128, 0), (128, 1)}, seen
+    # every K-major instantiation was visited by name: two tile configurations x {bfloat16, half} workspace, and the
+    # small configuration once more with the K-split
+    assert seen == {(256, 0, 0), (256, 1, 0), (128, 0, 0), (128, 1, 0), (128, 0, 1), (128, 1, 1)}, seen
     assert all_kernels > len(seen)
     # per k-tile: 4 k-steps x (FM + FN) fragments x 2 reads; the loop body appears at least once
-    assert all(reads_of[(256, f)] >= 4 * 6 * 2 for f in (0, 1)), reads_of
-    assert all(reads_of[(128, f)] >= 4 * 4 * 2 for f in (0, 1)), reads_of
+    assert all(reads_of[(256, f, 0)] >= 4 * 6 * 2 for f in (0, 1)), reads_of
+    assert all(reads_of[(128, f, k)] >= 4 * 4 * 2 for f in (0, 1) for k in (0, 1)), reads_of

@@ -483,3 +483,30 @@ def test_gram_side_tail_spiked_and_grouped(ns, gpu_device):
             single = ns.newton_schulz(x, O.QUINTIC, 1e-7, prec=prec, gram_tail=True)
             assert torch.equal(o, single), (prec, tuple(x.shape))
             assert _rel(o, O.newton_schulz(x.cpu(), O.QUINTIC, 1e-7, storage="fp32")) <= NS_TOL
+
+
+@pytest.mark.parametrize("shape", [(1536, 8192), (8192, 1536)])
+def test_k_split_of_long_reductions(ns, gpu_device, shape):
+    """A matrix with few upper-triangle tiles (21 of 256 x 256) and a long reduction (K = 8192) has its A = X X^T product
+    cut along K: four blocks per 128 x 128 quadrant leave fp32 partial results, the last one to arrive adds them in the
+    order of the parts.  The cut is a function of the matrix's own shape, so the matrix gives the same bits alone (the
+    small-call path), in a batch, in a grouped call next to other shapes, and on every repetition (which block arrives
+    last changes from run to run; the sum does not); and the result is within the bar of the fp32 oracle."""
+    G = _randn(shape, 77)
+    Gd = G.to(gpu_device)
+    want = O.newton_schulz(G, O.QUINTIC, 1e-7, storage="fp32")
+    for prec, bar in (("bf16", NS_TOL), ("f16", 4e-3)):
+        alone = ns.newton_schulz(Gd, O.QUINTIC, 1e-7, prec=prec)
+        torch.cuda.synchronize()
+        err = _rel(alone, want)
+        print("k-split", shape, prec, "rel err", err, flush=True)
+        assert err <= bar
+        for _ in range(3):
+            assert torch.equal(ns.newton_schulz(Gd, O.QUINTIC, 1e-7, prec=prec), alone)
+        batch = torch.stack([Gd, _randn(shape, 78).to(gpu_device), Gd])
+        out = ns.newton_schulz(batch, O.QUINTIC, 1e-7, prec=prec)
+        assert torch.equal(out[0], alone) and torch.equal(out[2], alone)
+        other = _randn((2, 256, 640), 79).to(gpu_device)
+        a, b = ns.newton_schulz_grouped([other, Gd], O.QUINTIC, 1e-7, prec=prec)
+        assert torch.equal(b, alone)
+        assert torch.equal(a, ns.newton_schulz(other, O.QUINTIC, 1e-7, prec=prec))
