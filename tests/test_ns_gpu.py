@@ -510,3 +510,23 @@ def test_k_split_of_long_reductions(ns, gpu_device, shape):
         a, b = ns.newton_schulz_grouped([other, Gd], O.QUINTIC, 1e-7, prec=prec)
         assert torch.equal(b, alone)
         assert torch.equal(a, ns.newton_schulz(other, O.QUINTIC, 1e-7, prec=prec))
+
+
+def test_odd_number_of_small_tiles_in_a_batch(ns, gpu_device):
+    """Short sides of 384 or 640 (three or five 128-tiles, the expert width of the depth-24 MoE set) and a ragged one, in
+    a batch large enough for the usual tile choice, in both orientations of the final store: within the bar of the fp32
+    oracle in either orientation (the two orientations sum the squares for the norm in different orders, so they agree
+    to the last bits only), and the same bits as a single call, which takes the small configuration throughout."""
+    for shape in [(384, 1024), (640, 768), (300, 1000)]:
+        G = _randn((24,) + shape, 41 + sum(shape))
+        out = ns.newton_schulz(G.to(gpu_device))
+        outT = ns.newton_schulz(G.mT.contiguous().to(gpu_device))
+        torch.cuda.synchronize()
+        assert _rel(outT.mT, out) <= 1e-3
+        for i in (0, 11, 23):
+            want = O.newton_schulz(G[i], O.QUINTIC, 1e-7, storage="fp32")
+            assert _rel(out[i], want) <= NS_TOL and _rel(outT[i].mT, want) <= NS_TOL, (shape, i)
+            assert torch.equal(ns.newton_schulz(G[i].to(gpu_device)), out[i])
+            assert torch.equal(ns.newton_schulz(G[i].mT.contiguous().to(gpu_device)), outT[i])
+        f16 = ns.newton_schulz(G.to(gpu_device), O.QUINTIC, 1e-7, prec="f16")
+        assert _rel(f16[5], O.newton_schulz(G[5], O.QUINTIC, 1e-7, storage="fp32")) <= 4e-3
