@@ -245,6 +245,8 @@ def main():
     ap.add_argument("--dump-launches", action="store_true", help="(debug) every timed launch of the instrumented step on stderr")
     ap.add_argument("--other-configs", default="1,3,4,5",
                     help="comma-separated benchmark configurations reported beside the headline (empty: none)")
+    ap.add_argument("--only-config", type=int, default=0, choices=[0, 1, 3, 4, 5],
+                    help="(profiling) run just this one of the other configurations and print its record instead of the headline line")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain device copy run once after the steps (yardstick for HBM byte counters)")
     args = ap.parse_args()
@@ -259,6 +261,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.only_config:
+        print(json.dumps({"only_config": args.only_config, **other_configs(dev, [args.only_config])}))
+        return
     params, grads = make_tensors(dev, args.seed, args.layers)
     for p, g in zip(params, grads):
         p.grad = g
