@@ -240,24 +240,37 @@ hipError_t launch_rounds(int tile, int mode, bool split, bool final_, const Grou
 static __device__ __align__(256) unsigned char scratch[MUON_NS_STATIC_SCRATCH_BYTES];
 
 namespace {
-std::mutex g_scratch_mutex;
-void* g_scratch_ptr[MAX_DEVICES] = {};
+// per device: the array's address, and what orders calls that come in on different streams (the event marks the end
+// of the last call's work; a call on another stream waits for it on the device, so two streams that share the array
+// take turns instead of racing).  Created once per device, on the first call.
+struct StaticScratch {
+  void* ptr = nullptr;
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool has_last = false;
+};
+std::mutex g_scratch_mutex;   // held while a call on the array is being enqueued
+StaticScratch g_scratch[MAX_DEVICES];
 
-// device address of `scratch` on the CURRENT device (looked up once per device)
-int static_scratch(void** out) {
+// the array of the CURRENT device (address looked up once per device); the caller holds g_scratch_mutex
+int static_scratch(StaticScratch** out) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= MAX_DEVICES) return MUON_E_UNSUPPORTED;
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (!g_scratch_ptr[dev]) {
+  StaticScratch& st = g_scratch[dev];
+  if (!st.ptr) {
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return (int)e;
     if (!ptr || ((uintptr_t)ptr & 255)) return MUON_E_WORKSPACE;
-    g_scratch_ptr[dev] = ptr;
+    hipEvent_t ev = nullptr;
+    e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+    if (e != hipSuccess) return (int)e;
+    st.done = ev;
+    st.ptr = ptr;
   }
-  *out = g_scratch_ptr[dev];
+  *out = &st;
   return 0;
 }
 }  // namespace
@@ -830,17 +843,37 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
 
 int muon_ns_batched_static(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld, void* out_dev,
                            int64_t out_batch_stride, int out_ld, int batch, int rows, int cols, const float* abc_host,
-                           int iters, float eps, int eps_mode, int prec_mode, int flags, void* stream) {
+                           int iters, float eps, int eps_mode, int prec_mode, int flags, void* stream_) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return MUON_E_ARG;
   if (prec_mode != MUON_PREC_BF16 && prec_mode != MUON_PREC_BF16_BSPLIT && prec_mode != MUON_PREC_F16) return MUON_E_ARG;
   if (plan_bytes_bound(batch, rows, cols, prec_mode) > (size_t)MUON_NS_STATIC_SCRATCH_BYTES) return MUON_E_STATIC_LIMIT;
-  void* ws = nullptr;
-  const int st = static_scratch(&ws);
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  StaticScratch* sc = nullptr;
+  const int st = static_scratch(&sc);
   if (st) return st;
+  // Calls on one stream are ordered by the stream.  A call on ANOTHER stream than the last one first waits (on the
+  // device) for the end of that call, so the two do not overlap on the array.  Not under stream capture: a captured call
+  // is replayed later, in an order that only the caller knows, and an event recorded outside the capture cannot be
+  // waited for inside it; replays that overlap other users of the array are the caller's to order.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  hipError_t e = hipStreamIsCapturing(stream, &capture);
+  if (e != hipSuccess) return (int)e;
+  const bool eager = capture == hipStreamCaptureStatusNone;
+  if (eager && sc->has_last && sc->last != stream && (e = hipStreamWaitEvent(stream, sc->done, 0)) != hipSuccess) return (int)e;
   // every byte of the workspace that a kernel reads is written earlier in the same call (the layout pass writes the
-  // zero padding, the products write whole tiles), so nothing left over from the previous call has to be cleared
-  return muon_ns_batched(in_dev, in_dtype, in_batch_stride, in_ld, out_dev, out_batch_stride, out_ld, batch, rows, cols,
-                         abc_host, iters, eps, eps_mode, prec_mode, flags, ws, MUON_NS_STATIC_SCRATCH_BYTES, stream);
+  // zero padding, the products write whole tiles, the K-split counters are cleared by a kernel), so nothing left over
+  // from the previous call has to be cleared
+  const int rc = muon_ns_batched(in_dev, in_dtype, in_batch_stride, in_ld, out_dev, out_batch_stride, out_ld, batch, rows,
+                                 cols, abc_host, iters, eps, eps_mode, prec_mode, flags, sc->ptr,
+                                 MUON_NS_STATIC_SCRATCH_BYTES, stream_);
+  if (eager) {
+    // (also after a failed call: some of its launches may be in flight)
+    if ((e = hipEventRecord(sc->done, stream)) != hipSuccess) return rc ? rc : (int)e;
+    sc->last = stream;
+    sc->has_last = true;
+  }
+  return rc;
 }
 
 size_t muon_syrk_workspace_bytes(int batch, int n, int k) {

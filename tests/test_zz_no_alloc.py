@@ -74,3 +74,63 @@ def test_static_scratch_rejects_what_does_not_fit(gpu_device):
     # bad extents are argument errors, as in muon_ns_batched
     abc = _lib.abc_array(coeffs)
     assert L.muon_ns_batched_static(x.data_ptr(), 0, 0, 0, out.data_ptr(), 0, 0, 0, 16, 16, abc, 5, 1e-7, 0, 0, 0, None) == -1
+
+
+def test_static_scratch_calls_on_two_streams_take_turns(gpu_device):
+    """Two streams that share the array without any host synchronisation between their calls: a call on another stream
+    than the last one waits on the device for the end of that one, so neither sees the other's iterates."""
+    from archscale_amd import _lib
+    L = _lib.lib()
+    coeffs = O.coefficient_schedule("quintic", 5)
+    xs = [_randn((4, 256, 640), 11).to(gpu_device), _randn((2, 384, 512), 12).to(gpu_device)]
+    want = []
+    for x in xs:
+        need = L.muon_ns_workspace_bytes(x.shape[0], x.shape[1], x.shape[2], _lib.PREC_BF16)
+        ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+        st, w = _call(L, _lib, "workspace", x, coeffs, _lib.PREC_BF16, ws=ws)
+        assert st == 0
+        want.append(w)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [None, None]
+    for rep in range(3):
+        for i in (0, 1, 1, 0):
+            with torch.cuda.stream(streams[i]):
+                st, got[i] = _call(L, _lib, "static", xs[i], coeffs, _lib.PREC_BF16)
+                assert st == 0, L.muon_status_string(st)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), rep
+
+
+def test_static_scratch_call_replays_in_a_graph(gpu_device):
+    """What the entry point is for: a call captured in a HIP graph (after one eager call, which looks the array up)
+    allocates nothing and replays; every replay, with eager work and synchronisations in between, equals the eager
+    result bit for bit (the input buffer is refilled before each replay)."""
+    from archscale_amd import _lib
+    L = _lib.lib()
+    coeffs = O.coefficient_schedule("quintic", 5)
+    shape = (3, 320, 1100)
+    x = _randn(shape, 21).to(gpu_device)
+    st, _ = _call(L, _lib, "static", x, coeffs, _lib.PREC_BF16)      # eager warm-up: address lookup happens here
+    assert st == 0
+    torch.cuda.synchronize()
+    out = torch.empty(shape, dtype=torch.bfloat16, device=gpu_device)
+    args = lambda stream: [x.data_ptr(), _lib.dtype_code(x.dtype), shape[1] * shape[2], shape[2], out.data_ptr(),
+                           shape[1] * shape[2], shape[2], shape[0], shape[1], shape[2], _lib.abc_array(coeffs), len(coeffs),
+                           1e-7, _lib.EPS_ADD, _lib.PREC_BF16, _lib.NS_CAST_INPUT_FIRST, stream]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = L.muon_ns_batched_static(*args(_lib.current_stream_ptr(gpu_device)))
+    assert st == 0, L.muon_status_string(st)
+    need = L.muon_ns_workspace_bytes(shape[0], shape[1], shape[2], _lib.PREC_BF16)
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+    for k in range(4):
+        x.copy_(_randn(shape, 30 + k).to(gpu_device))
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        st, want = _call(L, _lib, "workspace", x, coeffs, _lib.PREC_BF16, ws=ws)     # eager work between the replays
+        assert st == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), k
+    del graph
