@@ -32,7 +32,7 @@ NS_STATIC_SCRATCH_BYTES = 64 << 20
 STREAM_COPY, STREAM_READ, STREAM_MIX = 0, 1, 2
 E_STATIC_LIMIT = -4
 PROF_KEY_MOMENTUM_LAYOUT = 90000
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 #: numpy layouts of muon_pre_item / muon_post_item (natural C alignment)
 PRE_ITEM = np.dtype(
@@ -112,6 +112,7 @@ _SIGNATURES = {
         ctypes.POINTER(ctypes.c_float), ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "muon_ns_flops": (None, [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_double)] * 3),
+    "muon_ns_ksplit_info": (None, [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
     "muon_profile_begin": (ctypes.c_int, []),
     "muon_profile_collect": (ctypes.c_int, [
         ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_double),
@@ -283,6 +284,14 @@ def ns_flops(batch: int, rows: int, cols: int, iters: int, prec_mode: int) -> Tu
     d, s, i = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
     lib().muon_ns_flops(batch, rows, cols, iters, prec_mode, ctypes.byref(d), ctypes.byref(s), ctypes.byref(i))
     return d.value, s.value, i.value
+
+
+def ns_ksplit_info(rows: int, cols: int):
+    """((whole tiles, cut tiles, parts) for the reduction over the long side, the same for the short side) of one
+    rows x cols matrix: how the library cuts its symmetric products along K (parts == 1: not at all)."""
+    info = (ctypes.c_int * 6)()
+    lib().muon_ns_ksplit_info(rows, cols, info)
+    return tuple(info[:3]), tuple(info[3:])
 
 
 def profile_begin() -> None:

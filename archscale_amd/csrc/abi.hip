@@ -309,6 +309,15 @@ void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode, doub
   }
 }
 
+void muon_ns_ksplit_info(int rows, int cols, int* info) {
+  if (!info) return;
+  for (int i = 0; i < 6; ++i) info[i] = 0;
+  if (rows <= 0 || cols <= 0) return;
+  const SkShape s = sk_shape(rows < cols ? rows : cols, rows < cols ? cols : rows);
+  info[0] = s.long_k.full; info[1] = s.long_k.rem; info[2] = s.long_k.parts;
+  info[3] = s.short_k.full; info[4] = s.short_k.rem; info[5] = s.short_k.parts;
+}
+
 // plan + carved workspace pointers of one problem of a grouped call
 namespace {
 struct NsProblem {

@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define MUON_ABI_VERSION 2
+#define MUON_ABI_VERSION 3
 
 /* element types of caller tensors */
 #define MUON_DTYPE_BF16 0
@@ -111,8 +111,12 @@ int muon_ns_batched(const void* in_dev, int in_dtype, int64_t in_batch_stride, i
  * the process ends), and the call performs no hipMalloc / hipFree and calls no allocating library routine.
  * A problem whose muon_ns_workspace_bytes(batch, rows, cols, prec_mode) exceeds MUON_NS_STATIC_SCRATCH_BYTES is
  * rejected with MUON_E_STATIC_LIMIT before anything is launched.  All calls on one GPU share that GPU's array:
- * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered and safe.
- * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside a capture. */
+ * calls on one stream are ordered by the stream; a call on another stream than the previous one first waits, on the
+ * device, for the end of that one (an event that the library records after every eager call), so streams and host
+ * threads that share the array take turns.  A call under stream capture records and waits for nothing: replays of a
+ * captured call that overlap other users of the array on the same GPU race, and ordering them is the caller's job.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress) and creates that event; make that call
+ * outside a capture. */
 #define MUON_NS_STATIC_SCRATCH_BYTES (64u << 20)
 int muon_ns_batched_static(const void* in_dev, int in_dtype, int64_t in_batch_stride, int in_ld,
                            void* out_dev, int64_t out_batch_stride, int out_ld,
@@ -146,6 +150,16 @@ int muon_ns_grouped(const muon_ns_problem* problems_host, int n_problems,
  * authoritative count of what a call issued. */
 void muon_ns_flops(int batch, int rows, int cols, int iters, int prec_mode,
                    double* dense, double* symmetric, double* issued);
+
+/* How the symmetric products of ONE rows x cols matrix are cut along K (no counterpart in the reference; its Triton
+ * kernels take one program per output tile, lit_gpt/optim/newton_schulz_triton.py:51-53).  A matrix that leaves few
+ * upper-triangle tiles over after whole rounds of the chip and has a long reduction (K >= 8192) runs those leftover tiles
+ * as 128 x 128 quadrants with several blocks per quadrant, each over a part of K; the partial sums are added in the order
+ * of the parts, so the result is deterministic, and the rule looks at the matrix's own shape only, so a matrix gives
+ * the same bits alone and in any batch.  info (6 ints, HOST): for the reduction over the long side (A = X X^T) and
+ * then for the reduction over the short side (the m x m products): tiles of 256 x 256 that run whole, leftover tiles
+ * that are cut, parts per quadrant (1 = no cut).  muon_ns_workspace_bytes already includes the partial results. */
+void muon_ns_ksplit_info(int rows, int cols, int* info);
 
 /* Per-launch timing of the Newton-Schulz GEMM kernels, for roofline accounting (no counterpart in the
  * reference).  Between muon_profile_begin() and muon_profile_collect() every GEMM launch of muon_ns_batched is

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(handle, name), f"{name} is declared in the header but not exported"
     assert sorted(_lib.EXPORTED_SYMBOLS) == declared
-    assert handle.muon_abi_version() == _lib.ABI_VERSION == 2
+    assert handle.muon_abi_version() == _lib.ABI_VERSION == 3
     assert b"success" in handle.muon_status_string(0)
     assert b"workspace" in handle.muon_status_string(-2)
 
@@ -61,6 +61,31 @@ def test_struct_layouts_and_constants_match_header():
         assert ctypes.sizeof(cs) == nd.itemsize
         for name, _ in cs._fields_:
             assert getattr(cs, name).offset == nd.fields[name][1]
+
+
+def test_k_split_rule_is_a_function_of_the_shape():
+    """Which symmetric products are cut along K: none of the shapes that come in large batches (every class of the
+    depth-16 and depth-24 parameter sets, expert stacks), the leftover tiles of large single matrices with K >= 8192.
+    The workspace query includes the partial results."""
+    from archscale_amd import _lib
+    L = _lib.lib()
+    none = ((None, 0, 1), (None, 0, 1))
+    for shape in [(2048, 2048), (512, 2048), (5632, 2048), (2048, 5632), (3072, 3072), (768, 3072), (1536, 3072),
+                  (3072, 384), (256, 2048), (256, 8192), (1024, 8192), (4096, 4096), (100, 36)]:
+        lk, sk = _lib.ns_ksplit_info(*shape)
+        assert lk[1:] == none[0][1:] and sk[1:] == none[1][1:], shape
+    # 4096 x 14336: 16 * 17 / 2 = 136 tiles, all left over; only the reduction over the long side is long enough
+    assert _lib.ns_ksplit_info(4096, 14336) == ((0, 136, 4), (136, 0, 1))
+    assert _lib.ns_ksplit_info(14336, 4096) == _lib.ns_ksplit_info(4096, 14336)
+    # 8192 x 8192: 528 tiles = two whole rounds of 256 and 16 left over, both reductions have K = 8192
+    assert _lib.ns_ksplit_info(8192, 8192) == ((512, 16, 4), (512, 16, 4))
+    # 1536 x 8192: 21 tiles, K = 8192 over the long side only
+    assert _lib.ns_ksplit_info(1536, 8192) == ((0, 21, 4), (21, 0, 1))
+    # the partial results (64 KiB per quadrant and part) are part of the workspace
+    base = 2 * 4096 * 14336 * 2 + 2 * 4096 * 4096 * 2
+    need = L.muon_ns_workspace_bytes(1, 4096, 14336, 0)
+    assert need >= base + 136 * 4 * 4 * 65536 and need < base + 136 * 4 * 4 * 65536 + (8 << 20)
+    assert L.muon_ns_workspace_bytes(3, 4096, 14336, 0) >= 3 * (base + 136 * 4 * 4 * 65536)
 
 
 def test_workspace_and_flops_queries_need_no_gpu():
