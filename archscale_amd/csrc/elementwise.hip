@@ -398,8 +398,11 @@ hipError_t launch_layout_ptrs(const LayoutPtrs& ptrs, int n_mats, int in_dtype, 
 //     MOMLAY_MAX matrices of one shape (their tensors are separate allocations: pointers by value).
 // ---------------------------------------------------------------------------
 // tile of one block of the transposing pass: MOMLAY_TILE x MOMLAY_TILE elements (8 elements per thread and pass), so that
-// a row of it is 256 contiguous bytes in the source and in the transposed image.  Measured alternatives (64 x 256,
-// 256 x 64 and 32 x 512 tiles; the loads of all eight passes before the first store) were 5 to 20 % slower.
+// a row of it is 256 contiguous bytes in the source and in the transposed image.  Measured alternatives were 5 to 20 %
+// slower: 64 x 256, 256 x 64 and 32 x 512 tiles; the loads of all eight passes before the first store; and the transposed
+// store through LDS transpose reads (16-byte LDS writes, ds_read_b64_tr_b16), which leaves a wave writing 64 bytes to
+// each of 16 image rows per instruction instead of 256 bytes to each of 4 (4.75 against 5.26 TB/s): the stores, not
+// the 2-byte LDS accesses, are what this pass is sensitive to.
 constexpr int MOMLAY_TPR = MOMLAY_TILE / 8;          // threads per tile row (8 elements each)
 constexpr int MOMLAY_RPP = 256 / MOMLAY_TPR;         // tile rows per pass of the block
 constexpr int MOMLAY_PASSES = MOMLAY_TILE / MOMLAY_RPP;
