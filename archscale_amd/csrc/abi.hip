@@ -79,7 +79,8 @@ SkRule sk_rule(int tm, int KT) {
   const int T = (int)sym_tiles(tm);
   SkRule r = {T, 0, 1};
   const int full = T / 256 * 256, rem = T - full;
-  if (env_switches().ksplit == 0 || KT < SK_MIN_KT || rem < SK_MIN_REM) return r;
+  // (a tile configuration forced through the environment, a debugging switch, also switches the split off)
+  if (env_switches().ksplit == 0 || env_switches().tile != 0 || KT < SK_MIN_KT || rem < SK_MIN_REM) return r;
   int parts = SK_PARTS;
   if (env_switches().ksplit > 1 && KT / env_switches().ksplit >= 16) parts = env_switches().ksplit;   // (experiments)
   return SkRule{full, rem, parts};
