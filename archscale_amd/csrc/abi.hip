@@ -644,7 +644,14 @@ int ns_grouped_impl(const muon_ns_problem* problems_host, const muon_mns_problem
   // 1-2 % of accuracy (polar-express msign table, whose spectrum is not settled two iterations before the end:
   // 1.9e-3 -> 2.4e-3), so there the caller has to ask for it.
   const bool tail_wanted = (flags & MUON_NS_NO_GRAM_TAIL) ? false : ((flags & MUON_NS_GRAM_TAIL) ? true : !f16);
-  const bool tail = tail_wanted && normalize && !split_any && iters >= 3 && fold_ok(iters - 2) && fold_ok(iters - 1);
+  // (half storage holds B + aI times 2^6: with |A| <= 1.5 after the normalisation that is in range for any table whose
+  // last two rows keep 1.5 |b| + 2.25 |c| + |a| under 500 - every table of the reference is under 25; a custom table beyond
+  // that keeps its last iterations in bfloat16)
+  auto half_range_ok = [&](int it) {
+    return 1.5f * fabsf(abc_host[3 * it + 1]) + 2.25f * fabsf(abc_host[3 * it + 2]) + fabsf(abc_host[3 * it]) <= 500.f;
+  };
+  const bool tail = tail_wanted && normalize && !split_any && iters >= 3 && fold_ok(iters - 2) && fold_ok(iters - 1) &&
+                    half_range_ok(iters - 2) && half_range_ok(iters - 1);
   const int first_half_it = f16 ? (defer_all ? 1 : 0) : (tail ? iters - 2 : iters);
   // ---- Gram-side tail.  With P_k = a_k I + b_k A_k + c_k A_k^2 (symmetric, a polynomial in A_k = X_k X_k^T, so all of
   // them commute) the last two iterations are  X_N = P_N P_{N-1} X_{N-2}  with  A_{N-1} = P_{N-1} A_{N-2} P_{N-1}:

@@ -54,7 +54,8 @@ extern "C" {
                                       time */
 #define MUON_NS_NO_GRAM_TAIL 8      /* keep the last two iterations as plain iterations in the storage type of prec_mode */
 #define MUON_NS_GRAM_TAIL 16        /* take the tail described below also under MUON_PREC_F16 */
-/* The tail: a call with at least three iterations whose last two rows have |a| <= 4.2 (MUON_NS_NO_DIAG_FOLD not set,
+/* The tail: a call with at least three iterations whose last two rows have |a| <= 4.2 and 1.5 |b| + 2.25 |c| + |a| <= 500
+ * (the range of the half storage; every table of the reference is under 25) (MUON_NS_NO_DIAG_FOLD not set,
  * input normalised, no hi+lo pair) (1) keeps the matrices of the last two iterations in IEEE half also under
  * MUON_PREC_BF16, and (2) for every problem with long side >= 2 x short side finishes on the Gram side:
  * X_N = (P_N P_{N-1}) X_{N-2} with A_{N-1} = P_{N-1} A_{N-2} P_{N-1}, P = aI + bA + cA^2 - three m x m symmetric

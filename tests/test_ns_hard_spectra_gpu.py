@@ -122,3 +122,23 @@ def test_norm_below_epsilon_and_zero(gpu_device, prec):
     z = torch.zeros(3, 192, 448, dtype=torch.bfloat16, device=gpu_device)
     for tail in (None, False, True):
         assert torch.all(H.newton_schulz(z, O.QUINTIC, 1e-7, prec=prec, gram_tail=tail) == 0)
+
+
+def test_custom_table_beyond_the_half_range_keeps_bf16_storage(gpu_device):
+    """The half-storage tail assumes |B + aI| <= 1000 (it is stored times 2^6); every table of the reference is under 25.
+    A custom table whose last rows are beyond that (1.5 |b| + 2.25 |c| + |a| > 500) must not take the tail: the default
+    call equals the call with plain last iterations bit for bit, and stays finite where bf16 storage does."""
+    import archscale_amd.optim.newton_schulz_hip as H
+    g = torch.Generator().manual_seed(9)
+    G = torch.randn(64, 96, generator=g).to(torch.bfloat16).to(gpu_device)
+    mild = [(3.0, -3.2, 1.2)] * 3
+    for last in [(2.0, -400.0, 0.0), (1.0, 0.0, 300.0)]:
+        coeffs = mild + [last, last]
+        got = H.newton_schulz(G, coeffs, 1e-7)
+        plain = H.newton_schulz(G, coeffs, 1e-7, gram_tail=False)
+        torch.cuda.synchronize()
+        assert torch.equal(got, plain)
+        assert torch.isfinite(got.float()).all()
+    # a table inside the range still takes the tail by default (the two calls differ)
+    coeffs = mild + [(2.0, -1.5, 0.5)] * 2
+    assert not torch.equal(H.newton_schulz(G, coeffs, 1e-7), H.newton_schulz(G, coeffs, 1e-7, gram_tail=False))
