@@ -149,13 +149,40 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const int b = local / per_mat;
   int t = p.t_first + (local - b * per_mat);
   int ti, tj;
-  if (SYM) {
+  if (SYM && dM > 8 && (dM & 3) == 0) {
+    // A large upper triangle in blocks of 4 x 4 tiles, block row by block row (a diagonal block holds the 10 tiles of
+    // its own upper triangle): the 32 tiles that an XCD works on at a time are two neighbouring blocks, whose operand
+    // panels are 4 + 8 row panels of the one matrix.  Row by row a run would be one row panel against 32 others.
+    const int nb = dM >> 2;
+    int bi = 0, rowcount = 10 + (nb - 1) * 16;
+    while (t >= rowcount) { t -= rowcount; ++bi; rowcount -= 16; }
+    if (t < 10) {
+      const int i = (t >= 4) + (t >= 7) + (t >= 9);          // rows of the 4 x 4 triangle hold 4, 3, 2, 1 tiles
+      const int first = i == 0 ? 0 : i == 1 ? 4 : i == 2 ? 7 : 9;
+      ti = 4 * bi + i;
+      tj = 4 * bi + i + (t - first);
+    } else {
+      t -= 10;
+      const int bj = bi + 1 + (t >> 4), w = t & 15;
+      ti = 4 * bi + (w & 3);
+      tj = 4 * bj + (w >> 2);
+    }
+  } else if (SYM) {
     ti = 0;
     int rowlen = dM;
     while (t >= rowlen) { t -= rowlen; ++ti; --rowlen; }
     tj = ti + t;
+  } else if (dM > 8 && (dM & 3) == 0 && (dN & 3) == 0) {
+    // A wide tile grid in blocks of 4 x 4 tiles, the blocks of one block row (4 row panels of P) one after the other:
+    // the 32 tiles that an XCD works on at a time are two neighbouring blocks, 4 row panels of P and 8 of Q, 12 panels
+    // per k-step.  Whole columns of dM tiles at a time would stream dM + 32 / dM panels (33 for dM = 32).
+    const int blk = t >> 4, w = t & 15;
+    const int nbj = dN >> 2;
+    const int bi = blk / nbj, bj = blk - bi * nbj;
+    ti = 4 * bi + (w & 3);
+    tj = 4 * bj + (w >> 2);
   } else {
-    tj = t / dM;
+    tj = t / dM;   // up to 8 row panels: whole columns, 8 x 4 tiles per XCD for dM = 8
     ti = t - tj * dM;
   }
   if (gp.quarter) {
