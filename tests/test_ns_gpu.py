@@ -530,3 +530,22 @@ def test_odd_number_of_small_tiles_in_a_batch(ns, gpu_device):
             assert torch.equal(ns.newton_schulz(G[i].mT.contiguous().to(gpu_device)), outT[i])
         f16 = ns.newton_schulz(G.to(gpu_device), O.QUINTIC, 1e-7, prec="f16")
         assert _rel(f16[5], O.newton_schulz(G[5], O.QUINTIC, 1e-7, storage="fp32")) <= 4e-3
+
+
+@pytest.mark.parametrize("n", [3072, 2560, 4096])
+def test_large_triangles_are_covered_tile_by_tile(ns, gpu_device, n):
+    """The stand-alone symmetric products on matrices with more than eight tiles of 256 along a side (12, 10 and 16):
+    large upper triangles are walked in blocks of 4 x 4 tiles when the side is a multiple of four tiles (3072, 4096) and
+    row by row otherwise (2560); either way every tile must be written exactly as if it were computed alone.  The
+    result is checked against an fp32 product element by element (an unwritten tile holds whatever the workspace held,
+    a misplaced one the wrong block of the product) and it is bit-symmetric."""
+    X = _randn((n, 320), 51 + n, 0.05).to(gpu_device)
+    A = ns.ns_line_1(X)
+    want = X.float() @ X.float().T
+    torch.cuda.synchronize()
+    assert torch.equal(A, A.mT)
+    assert (A.float() - want).abs().max().item() <= 4e-3 * want.abs().max().item()
+    B = ns.ns_line_2(A, alpha=2.0315 / 64, beta=-4.775)
+    wantB = (2.0315 / 64) * (A.float() @ A.float()) - 4.775 * A.float()
+    assert torch.equal(B, B.mT)
+    assert (B.float() - wantB).abs().max().item() <= 6e-3 * wantB.abs().max().item()
