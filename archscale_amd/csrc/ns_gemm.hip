@@ -149,21 +149,24 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
   const int b = local / per_mat;
   int t = p.t_first + (local - b * per_mat);
   int ti, tj;
-  if (SYM && dM > 8 && (dM & 3) == 0) {
+  if (SYM && dM > 8) {
     // A large upper triangle in blocks of 4 x 4 tiles, block row by block row (a diagonal block holds the 10 tiles of
     // its own upper triangle): the 32 tiles that an XCD works on at a time are two neighbouring blocks, whose operand
     // panels are 4 + 8 row panels of the one matrix.  Row by row a run would be one row panel against 32 others.
-    const int nb = dM >> 2;
-    int bi = 0, rowcount = 10 + (nb - 1) * 16;
-    while (t >= rowcount) { t -= rowcount; ++bi; rowcount -= 16; }
-    if (t < 10) {
-      const int i = (t >= 4) + (t >= 7) + (t >= 9);          // rows of the 4 x 4 triangle hold 4, 3, 2, 1 tiles
-      const int first = i == 0 ? 0 : i == 1 ? 4 : i == 2 ? 7 : 9;
+    // The last block column is `last` (1 to 4) tiles wide, and the last diagonal block a triangle of that side.
+    const int nb = (dM + 3) >> 2, last = dM - 4 * (nb - 1);
+    int bi = 0, rowcount = 10 + (nb - 2) * 16 + 4 * last;
+    while (bi < nb - 1 && t >= rowcount) { t -= rowcount; ++bi; rowcount -= 16; }
+    const int side = bi == nb - 1 ? last : 4;
+    if (t < side * (side + 1) / 2) {
+      int i = 0, rowlen = side;                               // rows of the triangle hold side, side - 1, ... tiles
+      while (t >= rowlen) { t -= rowlen; ++i; --rowlen; }
       ti = 4 * bi + i;
-      tj = 4 * bi + i + (t - first);
+      tj = 4 * bi + i + t;
     } else {
       t -= 10;
-      const int bj = bi + 1 + (t >> 4), w = t & 15;
+      const int bj = bi + 1 + (t >> 4) < nb - 1 ? bi + 1 + (t >> 4) : nb - 1;
+      const int w = t - 16 * (bj - bi - 1);                   // 0 .. 4 x (width of block bj) - 1
       ti = 4 * bi + (w & 3);
       tj = 4 * bj + (w >> 2);
     }
@@ -172,15 +175,22 @@ ns_gemm_kernel(const GroupedGemmParams gp) {
     int rowlen = dM;
     while (t >= rowlen) { t -= rowlen; ++ti; --rowlen; }
     tj = ti + t;
-  } else if (dM > 8 && (dM & 3) == 0 && (dN & 3) == 0) {
+  } else if (dM > 8) {
     // A wide tile grid in blocks of 4 x 4 tiles, the blocks of one block row (4 row panels of P) one after the other:
     // the 32 tiles that an XCD works on at a time are two neighbouring blocks, 4 row panels of P and 8 of Q, 12 panels
-    // per k-step.  Whole columns of dM tiles at a time would stream dM + 32 / dM panels (33 for dM = 32).
-    const int blk = t >> 4, w = t & 15;
-    const int nbj = dN >> 2;
-    const int bi = blk / nbj, bj = blk - bi * nbj;
-    ti = 4 * bi + (w & 3);
-    tj = 4 * bj + (w >> 2);
+    // per k-step.  Whole columns of dM tiles at a time would stream dM + 32 / dM panels (33 for dM = 32, 24 for 22).
+    // The last block row and the last block of a row are as narrow as the grid leaves them (1 to 4 tiles).
+    const int nbi = (dM + 3) >> 2, nbj = (dN + 3) >> 2;
+    int bi = t / (4 * dN);
+    if (bi >= nbi) bi = nbi - 1;
+    const int r = t - bi * 4 * dN;
+    const int h = dM - 4 * bi < 4 ? dM - 4 * bi : 4;
+    int bj = r / (4 * h);
+    if (bj >= nbj) bj = nbj - 1;
+    const int q = r - bj * 4 * h;
+    const int qc = q / h;
+    ti = 4 * bi + (q - qc * h);
+    tj = 4 * bj + qc;
   } else {
     tj = t / dM;   // up to 8 row panels: whole columns, 8 x 4 tiles per XCD for dM = 8
     ti = t - tj * dM;

@@ -215,6 +215,27 @@ def test_single_step_without_normalisation(gpu_device, shape):
         newton_schulz_step_tsyrk(X.float().to(gpu_device), a, b, c)
 
 
+@pytest.mark.parametrize("shape", [(2304, 2560), (3328, 2816), (3584, 5632), (2560, 2560)])
+def test_wide_grids_whose_sides_are_not_multiples_of_four_tiles(gpu_device, shape):
+    """The product X' = (B + aI) X walks a grid of more than 8 tile rows (short side above 2048) in blocks of 4 x 4 tiles;
+    the last block row and the last block of a row are narrower when a side is no multiple of four tiles (grids of
+    9 x 10, 11 x 13, 14 x 22 and 10 x 10 tiles here; the symmetric products of the same step walk triangles of side 9,
+    11, 14 and 10).
+    A tile left out or written twice shows as an error of order one against the fp64 iteration."""
+    from archscale_amd.emerging.muon_utils import newton_schulz_step_tsyrk
+    print("case", shape, flush=True)
+    a, b, c = 3.4445, -4.7750, 2.0315
+    X = (_randn(shape, 15).float() / max(shape) ** 0.5 * 0.6).to(torch.bfloat16).to(gpu_device)
+    got = newton_schulz_step_tsyrk(X, a, b, c)
+    torch.cuda.synchronize()
+    Xd = X.double()
+    A = Xd @ Xd.T
+    want = a * Xd + (b * A + c * A @ A) @ Xd
+    assert _rel(got, want) <= 4e-3
+    err = (got.double() - want).abs()
+    assert err.max().item() <= 0.05 * want.abs().max().item()   # no tile missing: every entry is close, not just the norm
+
+
 def test_quartered_tail_matches_other_grids(ns, gpu_device):
     """A launch whose last round holds few tiles hands them to the 128x128 configuration as quadrants. Which tiles
     those are depends on the batch, the arithmetic of a tile does not: the same matrix gives the same bits alone
@@ -532,13 +553,14 @@ def test_odd_number_of_small_tiles_in_a_batch(ns, gpu_device):
         assert _rel(f16[5], O.newton_schulz(G[5], O.QUINTIC, 1e-7, storage="fp32")) <= 4e-3
 
 
-@pytest.mark.parametrize("n", [3072, 2560, 4096])
+@pytest.mark.parametrize("n", [3072, 2560, 4096, 2304, 2816, 3584])
 def test_large_triangles_are_covered_tile_by_tile(ns, gpu_device, n):
-    """The stand-alone symmetric products on matrices with more than eight tiles of 256 along a side (12, 10 and 16):
-    large upper triangles are walked in blocks of 4 x 4 tiles when the side is a multiple of four tiles (3072, 4096) and
-    row by row otherwise (2560); either way every tile must be written exactly as if it were computed alone.  The
-    result is checked against an fp32 product element by element (an unwritten tile holds whatever the workspace held,
-    a misplaced one the wrong block of the product) and it is bit-symmetric."""
+    """The stand-alone symmetric products on matrices with more than eight tiles of 256 along a side (12, 10, 16, 9, 11
+    and 14): large upper triangles are walked in blocks of 4 x 4 tiles; when the side is no multiple of four tiles the
+    last block column is 2, 1 or 3 tiles wide and the last diagonal block a triangle of that side.  Every tile must be
+    written exactly once.  The result is checked against an fp32 product element by element (an unwritten tile holds
+    whatever the workspace held, a misplaced one the wrong block of the product) and it is bit-symmetric."""
+    print("case", n, flush=True)
     X = _randn((n, 320), 51 + n, 0.05).to(gpu_device)
     A = ns.ns_line_1(X)
     want = X.float() @ X.float().T
